@@ -145,3 +145,80 @@ EIA_API int eia_splitk_act_and_mul(const float* part, int sk, int T, int F, void
   }
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// xIELU with two learned numbers (p, q) read from device memory (a weight reload needs no new
+// launch arguments):  z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z)
+// + z/2.  fp32 inside.  The input is a stored row [T, F] (type T, row stride ldx) or the fp32
+// split-K partials [sk, T, F] of the GEMM that produced it, summed here (F % 4 == 0 then).
+EIA_DEV float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
+EIA_DEV float xielu_f(float z, float ap, float aq) {
+  return z > 0.f ? ap * z * z + 0.5f * z : aq * (expm1f(z) - z) + 0.5f * z;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+xielu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ part, int sk,
+             const T* __restrict__ pq, T* __restrict__ out, long ldo, int rows, int F) {
+  const float ap = softplus_f(ld_f32<T>(pq, 0)), aq = 0.5f + softplus_f(ld_f32<T>(pq, 1));
+  if (part) {
+    const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (idx >= (long)rows * F) return;
+    const int row = idx / F, col = idx % F;
+    const long slab = (long)rows * F;
+    const float* p = part + idx;
+    f32x4 v = *reinterpret_cast<const f32x4*>(p);
+    for (int z = 1; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * slab);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st_f32<T>(out + (long)row * ldo, col + i, xielu_f(v[i], ap, aq));
+    return;
+  }
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)rows * F) return;
+  const int row = idx / F, col = idx % F;
+  st_f32<T>(out + (long)row * ldo, col, xielu_f(ld_f32<T>(x + (long)row * ldx, col), ap, aq));
+}
+
+EIA_API int eia_xielu(const void* x, long ldx, const float* part, int sk, const void* pq, void* out,
+                      long ldo, int rows, int F, int is_bf16, hipStream_t st) {
+  if (rows < 0 || F < 1 || !pq || !out || (x == nullptr) == (part == nullptr) ||
+      (part && (sk < 1 || F % 4)))
+    return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  const long n = part ? (long)rows * F / 4 : (long)rows * F;
+  dim3 grid((unsigned)((n + 255) / 256)), block(256);
+  if (is_bf16)
+    hipLaunchKernelGGL(xielu_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)x, ldx, part, sk,
+                       (const bf16_t*)pq, (bf16_t*)out, ldo, rows, F);
+  else
+    hipLaunchKernelGGL(xielu_kernel<float>, grid, block, 0, st, (const float*)x, ldx, part, sk,
+                       (const float*)pq, (float*)out, ldo, rows, F);
+  EIA_LAUNCH_CHECK();
+}
+
+// out[t, c] = a[t, c] * sigmoid(g[t, c]); a and g are rows with their own strides (either may be
+// a column slice of a wider row), fp32 inside.
+template <typename T>
+__global__ void __launch_bounds__(256)
+sigmoid_gate_kernel(const T* __restrict__ a, long lda, const T* __restrict__ g, long ldg,
+                    T* __restrict__ out, long ldo, int rows, int N) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long)rows * N) return;
+  const int row = idx / N, col = idx % N;
+  const float gv = ld_f32<T>(g + (long)row * ldg, col);
+  st_f32<T>(out + (long)row * ldo, col, ld_f32<T>(a + (long)row * lda, col) / (1.0f + expf(-gv)));
+}
+
+EIA_API int eia_sigmoid_gate(const void* a, long lda, const void* g, long ldg, void* out, long ldo,
+                             int rows, int N, int is_bf16, hipStream_t st) {
+  if (rows < 0 || N < 1 || !a || !g || !out) return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  dim3 grid((unsigned)(((long)rows * N + 255) / 256)), block(256);
+  if (is_bf16)
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)a, lda,
+                       (const bf16_t*)g, ldg, (bf16_t*)out, ldo, rows, N);
+  else
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, block, 0, st, (const float*)a, lda,
+                       (const float*)g, ldg, (float*)out, ldo, rows, N);
+  EIA_LAUNCH_CHECK();
+}

@@ -6,12 +6,31 @@
 //   score[h][j] = (q_abs[h] . c_j + rot(q_rot[h]) . k_rot_j) * scale
 //   lat[h] = sum_j softmax(score[h])_j c_j                (value up-projection by the caller)
 // every head reads the SAME cache rows, so a workgroup stages a key tile in LDS once and uses it
-// for all (query, head) rows it owns.  Scores, softmax weights and the accumulators are fp32;
-// activations are bf16 or fp32 (template T).
+// for all (query, head) rows it owns.  Options: a sliding window (position i sees j with
+// 0 <= i - j < window), a per-head sink (the softmax denominator also holds exp(sink[h]), which
+// has no key and no value and is not scaled), and the pair layout of the rotation ((2i, 2i+1) or
+// (i, i + rot_dims/2)) with a common factor on cos and sin.  Scores, softmax weights and the
+// accumulators are fp32; activations are bf16 or fp32 (template T).
 //
 //   eia_latent_prep : RMS-norm of the query latent, RMS-norm of c, rotation of k_rot, cache write
 //   eia_latent_attn : rotation of q_rot, tiled online-softmax attention, sigmoid head gate
 #include "eia_common.h"
+
+// Entry d (< rot_dims) of a vector after the rotation by position pos: src holds the unrotated
+// vector; pairs are (2i, 2i+1), or (i, i + rot_dims/2) when half; cos and sin are times amp.
+template <typename T>
+EIA_DEV float lat_rotated(const T* src, int d, int rot_dims, bool half, float amp, float pos,
+                          const float* __restrict__ inv_freq) {
+  const int hd = rot_dims >> 1;
+  const int i = half ? (d < hd ? d : d - hd) : (d >> 1);
+  const bool second = half ? d >= hd : (d & 1);
+  float sn, cs;
+  sincosf(pos * inv_freq[i], &sn, &cs);
+  sn *= amp;
+  cs *= amp;
+  const float u = ld_f32<T>(src, half ? i : 2 * i), w = ld_f32<T>(src, half ? i + hd : 2 * i + 1);
+  return second ? (w * cs + u * sn) : (u * cs - w * sn);
+}
 
 // ------------------------------------------------------------------------------------------ prep
 // fused [T, ld]: columns [q_off, q_off+q_rank) query latent, [c_off, c_off+R) KV latent,
@@ -24,7 +43,7 @@ latent_prep_kernel(const T* __restrict__ fused, long ld, int q_off, int q_rank,
                    const T* __restrict__ wc, int kr_off, int rd, int rot_dims,
                    const float* __restrict__ inv_freq, const int* __restrict__ positions,
                    const int* __restrict__ slot_mapping, T* __restrict__ cache, long cache_row,
-                   float eps) {
+                   float eps, int rot_half, float rot_amp) {
   __shared__ float scratch[2];
   const long t = blockIdx.x;
   const T* row = fused + t * ld;
@@ -52,14 +71,9 @@ latent_prep_kernel(const T* __restrict__ fused, long ld, int q_off, int q_rank,
     st_f32<T>(dst, c, ld_f32<T>(row, c_off + c) * inv * ld_f32<T>(wc, c));
   const float pos = (float)positions[t];
   for (int d = threadIdx.x; d < rd; d += blockDim.x) {
-    float v = ld_f32<T>(row, kr_off + d);
-    if (d < rot_dims) {
-      const int i = d >> 1;
-      float sn, cs;
-      sincosf(pos * inv_freq[i], &sn, &cs);
-      const float u = ld_f32<T>(row, kr_off + 2 * i), w = ld_f32<T>(row, kr_off + 2 * i + 1);
-      v = (d & 1) ? (w * cs + u * sn) : (u * cs - w * sn);
-    }
+    const float v = d < rot_dims
+        ? lat_rotated<T>(row + kr_off, d, rot_dims, rot_half != 0, rot_amp, pos, inv_freq)
+        : ld_f32<T>(row, kr_off + d);
     st_f32<T>(dst, R + d, v);
   }
 }
@@ -68,7 +82,7 @@ EIA_API int eia_latent_prep(const void* fused, long ld, int q_off, int q_rank, c
                             void* cq, long ldcq, int c_off, int R, const void* wc, int kr_off,
                             int rd, int rot_dims, const float* inv_freq, const int* positions,
                             const int* slot_mapping, void* cache, long cache_row, float eps,
-                            int T_, int is_bf16, hipStream_t st) {
+                            int rot_half, float rot_amp, int T_, int is_bf16, hipStream_t st) {
   if (T_ < 0 || q_rank < 0 || (cache && (R < 1 || rd < 0 || rot_dims > rd || (rot_dims & 1))))
     return EIA_BAD_SHAPE;
   if (T_ == 0) return EIA_OK;
@@ -76,12 +90,12 @@ EIA_API int eia_latent_prep(const void* fused, long ld, int q_off, int q_rank, c
     hipLaunchKernelGGL((latent_prep_kernel<bf16_t>), dim3(T_), dim3(128), 0, st,
                        (const bf16_t*)fused, ld, q_off, q_rank, (const bf16_t*)wq, (bf16_t*)cq,
                        ldcq, c_off, R, (const bf16_t*)wc, kr_off, rd, rot_dims, inv_freq, positions,
-                       slot_mapping, (bf16_t*)cache, cache_row, eps);
+                       slot_mapping, (bf16_t*)cache, cache_row, eps, rot_half, rot_amp);
   else
     hipLaunchKernelGGL((latent_prep_kernel<float>), dim3(T_), dim3(128), 0, st,
                        (const float*)fused, ld, q_off, q_rank, (const float*)wq, (float*)cq, ldcq,
                        c_off, R, (const float*)wc, kr_off, rd, rot_dims, inv_freq, positions,
-                       slot_mapping, (float*)cache, cache_row, eps);
+                       slot_mapping, (float*)cache, cache_row, eps, rot_half, rot_amp);
   EIA_LAUNCH_CHECK();
 }
 
@@ -101,6 +115,9 @@ struct LatentAttnArgs {
   const void* gate; long gate_st;           // nullable: sigmoid(gate[t][h]) scales head h
   void* out; long out_st, out_sh;           // (t, h, r)
   float scale; int H, R, rd, bs, QB, HB, KC, ldk;
+  int window;                               // > 0: position i sees j with 0 <= i - j < window
+  const float* sink;                        // nullable [H]: exp(sink[h]) joins the denominator
+  int rot_half; float rot_amp;              // pair layout and cos / sin factor of the rotation
   // MFMA decode only: the keys of a row split over grid.z partitions; each writes its
   // unnormalised accumulators and (running max in log2 units, sum) for the merge kernel
   int nparts; float* part_acc; float* part_ml;
@@ -150,14 +167,10 @@ latent_attn_kernel(LatentAttnArgs a) {
       } else {
         const int dd = d - a.R;
         const T* src = qr + row * a.qr_st + h * a.qr_sh;
-        v = ld_f32<T>(src, dd);
-        if (dd < a.rot_dims) {
-          const int i = dd >> 1;
-          float sn, cs;
-          sincosf((float)a.positions[row] * a.inv_freq[i], &sn, &cs);
-          const float u = ld_f32<T>(src, 2 * i), w = ld_f32<T>(src, 2 * i + 1);
-          v = (dd & 1) ? (w * cs + u * sn) : (u * cs - w * sn);
-        }
+        v = dd < a.rot_dims
+            ? lat_rotated<T>(src, dd, a.rot_dims, a.rot_half != 0, a.rot_amp,
+                             (float)a.positions[row], a.inv_freq)
+            : ld_f32<T>(src, dd);
       }
       v *= a.scale;
     }
@@ -172,10 +185,11 @@ latent_attn_kernel(LatentAttnArgs a) {
 #pragma unroll
   for (int i = 0; i < LAT_ACC_MAX; ++i) acc[i] = 0.f;
   const int nacc = (M * a.R + 255) >> 8;
-  const int kmax = a.positions[row0 + ntok - 1] + 1;     // keys 0..kmax-1 are visible to the tile
+  const int kmax = a.positions[row0 + ntok - 1] + 1;     // keys kmin..kmax-1 are visible to the tile
+  const int kmin = a.window > 0 ? max(0, a.positions[row0] - a.window + 1) : 0;
   __syncthreads();
 
-  for (int k0 = 0; k0 < kmax; k0 += KC) {
+  for (int k0 = kmin; k0 < kmax; k0 += KC) {
     // key tile -> LDS
     for (int e = tid; e < KC * Dk; e += 256) {
       const int j = e / Dk, d = e - j * Dk;
@@ -194,7 +208,8 @@ latent_attn_kernel(LatentAttnArgs a) {
       const int t = m / a.HB;
       const int kp = k0 + j;
       float s = -INFINITY;
-      if (t < ntok && kp <= a.positions[row0 + t]) {
+      if (t < ntok && kp <= a.positions[row0 + t] &&
+          (a.window <= 0 || a.positions[row0 + t] - kp < a.window)) {
         const float* q = qs + (long)m * Dk;
         const T* k = kt + (long)j * ldk;
         s = 0.f;
@@ -254,7 +269,9 @@ latent_attn_kernel(LatentAttnArgs a) {
         const int t = m / a.HB, h = h0 + (m - t * a.HB);
         if (t < ntok && h < a.H) {
           const long row = row0 + t;
-          float v = acc[i] / lrow[m];
+          float l = lrow[m];
+          if (a.sink) l += expf(a.sink[h] - mrow[m]);
+          float v = acc[i] / l;
           if (gate) v *= 1.0f / (1.0f + expf(-ld_f32<T>(gate, row * a.gate_st + h)));
           st_f32<T>(out, row * a.out_st + h * a.out_sh + r, v);
         }
@@ -271,7 +288,8 @@ EIA_API int eia_latent_attn(const void* qa, long qa_st, long qa_sh, const void* 
                             const int* seq_lens, const int* cu_q, const int* work, int n_items,
                             const int* positions, const void* gate, long gate_st, void* out,
                             long out_st, long out_sh, float scale, int H, int R, int rd, int bs,
-                            int QB, int is_bf16, hipStream_t st) {
+                            int QB, int window, const float* sink, int rot_half, float rot_amp,
+                            int is_bf16, hipStream_t st) {
   if (H < 1 || R < 1 || rd < 0 || bs < 1 || QB < 1 || rot_dims > rd || (rot_dims & 1) ||
       cache_row < R + rd || (cu_q && !work))
     return EIA_BAD_SHAPE;
@@ -295,7 +313,8 @@ EIA_API int eia_latent_attn(const void* qa, long qa_st, long qa_sh, const void* 
   if (lds > 150 * 1024) return EIA_UNSUPPORTED;
   LatentAttnArgs a{qa, qa_st, qa_sh, qr, qr_st, qr_sh, inv_freq, rot_dims, cache, cache_row,
                    block_table, bt_stride, seq_lens, cu_q, work, n_items, positions, gate, gate_st,
-                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, KC, ldk, 1, nullptr, nullptr};
+                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, KC, ldk, window, sink, rot_half,
+                   rot_amp, 1, nullptr, nullptr};
   dim3 grid(n_items, (H + HB - 1) / HB);
   if (is_bf16) {
     if (lds > 48 * 1024)
@@ -379,14 +398,10 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
             v = bf2f(qa[d]);
           } else {
             const int dd = d - a.R;
-            v = bf2f(qr[dd]);
-            if (dd < a.rot_dims) {
-              const int i = dd >> 1;
-              float sn, cs;
-              sincosf((float)qpos * a.inv_freq[i], &sn, &cs);
-              const float u = bf2f(qr[2 * i]), w = bf2f(qr[2 * i + 1]);
-              v = (dd & 1) ? (w * cs + u * sn) : (u * cs - w * sn);
-            }
+            v = dd < a.rot_dims
+                ? lat_rotated<bf16_t>(qr, dd, a.rot_dims, a.rot_half != 0, a.rot_amp, (float)qpos,
+                                      a.inv_freq)
+                : bf2f(qr[dd]);
           }
         }
         qf[s][e] = f2bf(v);
@@ -401,13 +416,16 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
   float mrun = -INFINITY, lrun = 0.f;
   const float scale_log2 = a.scale * 1.4426950408889634f;
   const int kmax = a.positions[row0 + ntok - 1] + 1;
-  int k_begin = 0, k_end = kmax;
+  // first 32-key unit that holds a key some row of the tile sees
+  const int kmin = a.window > 0 ? (max(0, a.positions[row0] - a.window + 1) & ~31) : 0;
+  int k_begin = kmin, k_end = kmax;
   if (a.nparts > 1) {                                      // this partition's run of 32-key units
-    const int units = (kmax + 31) >> 5;
+    const int units = (kmax - kmin + 31) >> 5;
     const int per = (units + a.nparts - 1) / a.nparts;
-    k_begin = min((int)blockIdx.z * per, units) << 5;
-    k_end = min(kmax, ((int)blockIdx.z + 1) * per << 5);
+    k_begin = kmin + (min((int)blockIdx.z * per, units) << 5);
+    k_end = min(kmax, kmin + (((int)blockIdx.z + 1) * per << 5));
   }
+  const int wlo = a.window > 0 ? qpos - a.window + 1 : 0;   // first key this lane's row sees
   const int cpr = Dkp >> 3;                                // 16-byte chunks per (padded) key row
   const int nchunk = 32 * cpr;
 
@@ -475,8 +493,8 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int ka = k0 + 8 * g + i, kb = ka + 4;
-      v[i] = (ka <= qpos) ? s0[i] * scale_log2 : -INFINITY;
-      v[4 + i] = (kb <= qpos) ? s1[i] * scale_log2 : -INFINITY;
+      v[i] = (ka <= qpos && ka >= wlo) ? s0[i] * scale_log2 : -INFINITY;
+      v[4 + i] = (kb <= qpos && kb >= wlo) ? s1[i] * scale_log2 : -INFINITY;
     }
     float mloc = v[0];
 #pragma unroll
@@ -535,6 +553,7 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
     }
     return;
   }
+  if (a.sink) lrun += exp2f(a.sink[h] * 1.4426950408889634f - mrun);
   float f = 1.0f / lrun;
   if (a.gate) {
     const bf16_t* gate = static_cast<const bf16_t*>(a.gate);
@@ -559,7 +578,8 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
 __global__ void __launch_bounds__(128)
 latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                     int nparts, const int* __restrict__ seq_lens, const bf16_t* __restrict__ gate,
-                    long gate_st, bf16_t* __restrict__ out, long out_st, long out_sh, int H, int R) {
+                    long gate_st, const float* __restrict__ sink, bf16_t* __restrict__ out,
+                    long out_st, long out_sh, int H, int R) {
   const int row = blockIdx.x, h = blockIdx.y;
   if (seq_lens && seq_lens[row] <= 0) return;
   const long pr = ((long)row * H + h) * nparts;
@@ -570,6 +590,7 @@ latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict_
     const float m = part_ml[2 * (pr + p)];
     if (m != -INFINITY) L += part_ml[2 * (pr + p) + 1] * exp2f(m - M);
   }
+  if (sink && M != -INFINITY) L += exp2f(sink[h] * 1.4426950408889634f - M);
   float f = L > 0.f ? 1.0f / L : 0.f;
   if (gate) f *= 1.0f / (1.0f + expf(-bf2f(gate[row * gate_st + h])));
   for (int c = threadIdx.x; c < R; c += blockDim.x) {
@@ -596,6 +617,7 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
                                  const int* work, int n_items, const int* positions,
                                  const void* gate, long gate_st, void* out, long out_st,
                                  long out_sh, float scale, int H, int R, int rd, int bs, int QB,
+                                 int window, const float* sink, int rot_half, float rot_amp,
                                  int nparts, float* part_acc, float* part_ml, hipStream_t st) {
   if (H < 1 || R < 1 || rd < 0 || bs < 1 || QB < 1 || rot_dims > rd || (rot_dims & 1) ||
       cache_row < R + rd || (cu_q && !work))
@@ -614,8 +636,8 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
   const size_t lds = ((size_t)32 * ldk + (size_t)nc * 16 * 40) * 2;
   LatentAttnArgs a{qa, qa_st, qa_sh, qr, qr_st, qr_sh, inv_freq, rot_dims, cache, cache_row,
                    block_table, bt_stride, seq_lens, cu_q, work, n_items, positions, gate, gate_st,
-                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, 32, ldk, nparts, part_acc,
-                   part_ml};
+                   out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, 32, ldk, window, sink, rot_half,
+                   rot_amp, nparts, part_acc, part_ml};
   dim3 grid(n_items, (H + HB - 1) / HB, nparts);
 #define LAT_MFMA(NK, NC, SV)                                                                \
   do {                                                                                      \
@@ -637,7 +659,7 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
 #undef LAT_MFMA
   if (nparts > 1)
     hipLaunchKernelGGL(latent_merge_kernel, dim3(n_items, H), dim3(128), 0, st, part_acc, part_ml,
-                       nparts, seq_lens, static_cast<const bf16_t*>(gate), gate_st,
+                       nparts, seq_lens, static_cast<const bf16_t*>(gate), gate_st, sink,
                        static_cast<bf16_t*>(out), out_st, out_sh, H, R);
   EIA_LAUNCH_CHECK();
 }

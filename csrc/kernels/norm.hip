@@ -399,3 +399,98 @@ EIA_API int eia_gnorm(const void* y, long ldy, const float* ypart, int sk, const
 #undef GNORM_LAUNCH
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Boundary of a layer whose sublayers run side by side on one normed input, around an fp32
+// residual stream.  One launch does, per row,
+//   x += y1 + y2                              (each given or not: sublayer outputs, un-normed)
+//   h  = x / sqrt(mean(x^2) + eps) * w_next   (h != nullptr: the next layer's input)
+// Each y is a stored row (type T, row stride ld) or the fp32 split-K partials [sk, rows, W] of the
+// GEMM that produced it (+ bias), summed here.  A thread re-reads only the columns it wrote, so
+// the row needs no barrier besides the one inside the sum of squares.
+template <typename T> struct AddRmsSrc {
+  const T* y; long ld; const float* part; int sk; const T* bias;
+};
+template <typename T>
+EIA_DEV f32x4 add_rms_load(const AddRmsSrc<T>& s, long row, int c, long pstride, int W) {
+  f32x4 v = {0.f, 0.f, 0.f, 0.f};
+  if (s.y) {
+    v = ld4_f32<T>(s.y + row * s.ld + c);
+  } else if (s.part) {
+    if (s.bias) v = ld4_f32<T>(s.bias + c);
+    const float* p = s.part + row * (long)W + c;
+#pragma unroll 4
+    for (int z = 0; z < s.sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * pstride);
+  }
+  return v;
+}
+
+template <typename T, bool VEC>
+__global__ void __launch_bounds__(256)
+add_rms_kernel(AddRmsSrc<T> s1, AddRmsSrc<T> s2, float* __restrict__ x,
+               const T* __restrict__ w_next, T* __restrict__ h, long ldh, float eps, int W,
+               long pstride) {
+  __shared__ float scratch[4];
+  const long row = blockIdx.x;
+  float* xr = x + row * (long)W;
+  const bool any = s1.y || s1.part || s2.y || s2.part;
+  float ss = 0.f;
+  if constexpr (VEC) {
+    for (int c = 4 * threadIdx.x; c < W; c += 4 * blockDim.x) {
+      f32x4 xv = *reinterpret_cast<f32x4*>(xr + c);
+      if (any) {
+        xv += add_rms_load<T>(s1, row, c, pstride, W) + add_rms_load<T>(s2, row, c, pstride, W);
+        *reinterpret_cast<f32x4*>(xr + c) = xv;
+      }
+      ss += sumsq4(xv);
+    }
+  } else {
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      float xv = xr[c];
+      if (s1.y) xv += ld_f32<T>(s1.y + row * s1.ld, c);
+      if (s2.y) xv += ld_f32<T>(s2.y + row * s2.ld, c);
+      if (any) xr[c] = xv;
+      ss += xv * xv;
+    }
+  }
+  if (!h) return;
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)W + eps);
+  if constexpr (VEC) {
+    for (int c = 4 * threadIdx.x; c < W; c += 4 * blockDim.x)
+      st4_f32<T>(h + row * ldh + c,
+                 *reinterpret_cast<const f32x4*>(xr + c) * inv * ld4_f32<T>(w_next + c));
+  } else {
+    for (int c = threadIdx.x; c < W; c += blockDim.x)
+      st_f32<T>(h + row * ldh, c, xr[c] * inv * ld_f32<T>(w_next, c));
+  }
+}
+
+// x fp32 [rows, W] contiguous; y1 / y2, their biases, w_next and h are bf16 when is_bf16 else
+// fp32.  Partials need W % 4 == 0.
+EIA_API int eia_add_rms(const void* y1, long ld1, const float* p1, int sk1, const void* b1,
+                        const void* y2, long ld2, const float* p2, int sk2, const void* b2,
+                        float* x, const void* w_next, void* h, long ldh, float eps, int rows, int W,
+                        int is_bf16, hipStream_t st) {
+  if (rows < 0 || W < 1 || !x || (h && !w_next) || (y1 && p1) || (y2 && p2) ||
+      (p1 && (sk1 < 1 || W % 4)) || (p2 && (sk2 < 1 || W % 4)))
+    return EIA_BAD_SHAPE;
+  if (rows == 0) return EIA_OK;
+  const bool vec = W % 4 == 0 && ld1 % 4 == 0 && ld2 % 4 == 0 && ldh % 4 == 0;
+  if (!vec && (p1 || p2)) return EIA_BAD_SHAPE;
+  const int threads = W >= 1024 ? 256 : (W >= 512 ? 128 : 64);
+  const long ps = (long)rows * W;
+#define ADD_RMS_LAUNCH(TT, VV)                                                                  \
+  do {                                                                                          \
+    AddRmsSrc<TT> a{(const TT*)y1, ld1, p1, sk1, (const TT*)b1};                                \
+    AddRmsSrc<TT> b{(const TT*)y2, ld2, p2, sk2, (const TT*)b2};                                \
+    hipLaunchKernelGGL((add_rms_kernel<TT, VV>), dim3(rows), dim3(threads), 0, st, a, b, x,     \
+                       (const TT*)w_next, (TT*)h, ldh, eps, W, ps);                             \
+  } while (0)
+  if (is_bf16) {
+    if (vec) ADD_RMS_LAUNCH(bf16_t, true); else ADD_RMS_LAUNCH(bf16_t, false);
+  } else {
+    if (vec) ADD_RMS_LAUNCH(float, true); else ADD_RMS_LAUNCH(float, false);
+  }
+#undef ADD_RMS_LAUNCH
+  EIA_LAUNCH_CHECK();
+}

@@ -11,6 +11,8 @@
 //   s_h    = sum_g talk[h, g] * raw_g                             (talk == nullptr: s = raw)
 //   visible: j <= i and (i - j < window or j < keep)              (window <= 0: every j <= i)
 //   p      = softmax over the visible keys, per map;  a_m = sum_j p_mj v_j
+//   wmode 1: p = sigmoid(s_m + bias[m]) for every visible key, not normalised over the keys
+//            (bias == nullptr: 0; no head mixing, P == 1)
 //
 // Epilogue 0: out[h] = a_h * sigmoid(gate[h])   (gate == nullptr: out = a; P must be 1)
 // Epilogue 1: o = a_{2h} - lam * a_{2h+1};  out[h] = o / sqrt(mean(o^2) + eps) * post   (P == 2;
@@ -112,6 +114,113 @@ EIA_API int eia_qk_norm_cache(const void* fused, long ld, const float* part, int
 }
 
 // ---------------------------------------------------------------------------------------------
+// Cache write for heads that are normed as ONE vector and then rotated.  One workgroup per token:
+//   q columns [MQ * D] -> divided by their common root mean square, times qw[MQ * D] (qw == null:
+//                         no norm) -> rotation of the first rot_dims entries of every head
+//                         -> q_out[t, MQ * D]
+//   k columns [MK * D] -> the same with kw -> key row of the token's slot
+//   values             -> copied as projected -> value columns of the slot (page-transposed)
+// Rotation of head entry d < rot_dims at position p: pairs (2i, 2i+1), or (i, i + rot_dims/2) when
+// half; angle p * inv_freq[i] in fp32; cos and sin times amp.  Slots < 0 write no cache rows.
+// The row is stored (fused) or still the fp32 split-K partials of the projection GEMM (+ bias).
+template <typename T>
+__global__ void __launch_bounds__(256)
+qk_rope_cache_kernel(const T* __restrict__ fused, long ld, const float* __restrict__ part, int sk,
+                     long pstride, const T* __restrict__ bias, int q_off, int k_off, int v_off,
+                     int MQ, int MK, int D, int VW, const T* __restrict__ qw,
+                     const T* __restrict__ kw, const float* __restrict__ inv_freq, int rot_dims,
+                     int half, float amp, const int* __restrict__ positions, T* __restrict__ q_out,
+                     long ldq, T* __restrict__ kc, T* __restrict__ vc,
+                     const int* __restrict__ slots, int bs, float eps) {
+  __shared__ float scratch[4];
+  const long t = blockIdx.x;
+  const long slot = slots ? (long)slots[t] : -1;
+  extern __shared__ float rsum[];                   // [ld] when the row arrives as partials
+  if (part) {
+    for (int c = 4 * threadIdx.x; c < (int)ld; c += 4 * blockDim.x) {
+      f32x4 v = {0.f, 0.f, 0.f, 0.f};
+      if (bias) v = f32x4{ld_f32<T>(bias, c), ld_f32<T>(bias, c + 1), ld_f32<T>(bias, c + 2),
+                          ld_f32<T>(bias, c + 3)};
+      const float* p = part + t * ld + c;
+#pragma unroll 8
+      for (int z = 0; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * pstride);
+      *reinterpret_cast<f32x4*>(rsum + c) = v;
+    }
+    __syncthreads();
+  }
+  auto val = [&](int c) -> float { return fused ? ld_f32<T>(fused + t * ld, c) : rsum[c]; };
+  const float pos = (float)positions[t];
+  const int hd = rot_dims >> 1;
+  for (int side = 0; side < 2; ++side) {
+    if (side == 1 && slot < 0) break;               // (uniform per workgroup)
+    const int n = (side ? MK : MQ) * D, off = side ? k_off : q_off;
+    const T* w = side ? kw : qw;
+    float inv = 1.f;
+    if (w) {
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < n; c += blockDim.x) {
+        const float v = val(off + c);
+        ss += v * v;
+      }
+      inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)n + eps);
+    }
+    T* dst = side ? kc + slot * (long)n : q_out + t * ldq;
+    auto normed = [&](int c) -> float {
+      return val(off + c) * inv * (w ? ld_f32<T>(w, c) : 1.f);
+    };
+    for (int c = threadIdx.x; c < n; c += blockDim.x) {
+      const int d = c % D, c0 = c - d;
+      float v = normed(c);
+      if (d < rot_dims) {
+        const int i = half ? (d < hd ? d : d - hd) : (d >> 1);
+        const bool second = half ? d >= hd : (d & 1);
+        float sn, cs;
+        sincosf(pos * inv_freq[i], &sn, &cs);
+        sn *= amp;
+        cs *= amp;
+        const int da = half ? i : 2 * i, db = half ? i + hd : 2 * i + 1;
+        const float o = normed(c0 + (second ? da : db));    // the pair's other entry
+        v = second ? (v * cs + o * sn) : (v * cs - o * sn);
+      }
+      st_f32<T>(dst, c, v);
+    }
+  }
+  if (slot >= 0) {
+    T* dst = vc + (slot / bs) * (long)VW * bs + slot % bs;
+    for (int c = threadIdx.x; c < VW; c += blockDim.x) st_f32<T>(dst, (long)c * bs, val(v_off + c));
+  }
+}
+
+EIA_API int eia_qk_rope_cache(const void* fused, long ld, const float* part, int sk,
+                              const void* bias, int q_off, int k_off, int v_off, int MQ, int MK,
+                              int D, int VW, const void* qw, const void* kw, const float* inv_freq,
+                              int rot_dims, int half, float amp, const int* positions, void* q_out,
+                              long ldq, void* kc, void* vc, const int* slots, int bs, float eps,
+                              int T, int is_bf16, hipStream_t st) {
+  if (T < 0 || MQ < 1 || MK < 1 || D < 1 || VW < 1 || bs < 1 || !q_out || !kc || !vc || !positions ||
+      rot_dims < 0 || rot_dims > D || (rot_dims & 1) || (rot_dims && !inv_freq) ||
+      (fused == nullptr) == (part == nullptr) || (part && (sk < 1 || ld % 4)))
+    return EIA_BAD_SHAPE;
+  if (T == 0) return EIA_OK;
+  const long ps = (long)T * ld;
+  const size_t lds = part ? sizeof(float) * ld : 0;
+  if (lds > 64 * 1024) return EIA_UNSUPPORTED;
+  if (is_bf16)
+    hipLaunchKernelGGL((qk_rope_cache_kernel<bf16_t>), dim3(T), dim3(256), lds, st,
+                       (const bf16_t*)fused, ld, part, sk, ps, (const bf16_t*)bias, q_off, k_off,
+                       v_off, MQ, MK, D, VW, (const bf16_t*)qw, (const bf16_t*)kw, inv_freq,
+                       rot_dims, half, amp, positions, (bf16_t*)q_out, ldq, (bf16_t*)kc,
+                       (bf16_t*)vc, slots, bs, eps);
+  else
+    hipLaunchKernelGGL((qk_rope_cache_kernel<float>), dim3(T), dim3(256), lds, st,
+                       (const float*)fused, ld, part, sk, ps, (const float*)bias, q_off, k_off,
+                       v_off, MQ, MK, D, VW, (const float*)qw, (const float*)kw, inv_freq, rot_dims,
+                       half, amp, positions, (float*)q_out, ldq, (float*)kc, (float*)vc, slots, bs,
+                       eps);
+  EIA_LAUNCH_CHECK();
+}
+
+// ---------------------------------------------------------------------------------------------
 struct WinAttnArgs {
   const void* q; long ldq;          // [rows, M * D]
   const void* kc; const void* vc;   // [blocks, bs, G * P * D], [blocks, G * Dv, bs]
@@ -131,6 +240,8 @@ struct WinAttnArgs {
   int nparts;                       // MFMA form: key partitions over grid.z (1: none)
   int raw_bufs;                     // MFMA form with head mixing: raw-score buffers in LDS (1, 2)
   float* part_acc; float* part_ml;  // [rows, M, nparts, Dv] and [rows, M, nparts, 2] partials
+  int wmode;                        // 0: softmax; 1: sigmoid(score + bias), un-normalised
+  const float* bias;                // [M] or null (wmode 1)
 };
 
 // The visible keys of a 16-query tile as absolute 32-key blocks: the blocks of the kept first
@@ -238,6 +349,12 @@ window_attn_kernel(const WinAttnArgs a) {
         } else {
           s = sraw[m * WA_KT + lane];
         }
+        if (a.wmode == 1) {                            // plain sigmoid weights: nothing to rescale
+          const float z = s + (a.bias ? a.bias[m] : 0.f);
+          pw[m * WA_KT + lane] = valid ? 1.0f / (1.0f + expf(-z)) : 0.f;
+          if (lane == 0) { alpha[m] = 1.f; lrun[m] = 1.f; }
+          continue;
+        }
         if (!valid) s = -INFINITY;
         const float mo = mrun[m];
         const float mn = fmaxf(mo, wave_max(s));
@@ -314,21 +431,21 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
                             const float* talk, const void* gate, long ldg, void* out, long ldo,
                             int H, int G, int P, int D, int Dv, int bs, int window, int keep,
                             int qb, int epilogue, const float* lam, float eps, float post,
-                            int is_bf16,
-                            hipStream_t st) {
+                            int wmode, const float* bias, int is_bf16, hipStream_t st) {
   if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || D < 1 || Dv < 1 || bs < 1 ||
       keep < 0 || qb < 1 || !q || !kc || !vc || !bt || !positions || !mult || !out)
     return EIA_BAD_SHAPE;
   if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
   if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam)))
     return EIA_BAD_SHAPE;
+  if ((wmode != 0 && wmode != 1) || (wmode == 1 && (talk || P != 1))) return EIA_BAD_SHAPE;
   const int M = H * P;
   const size_t lds = wa_lds_bytes(M, D, Dv);
   if (M * Dv > 256 * WA_ACC || lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
                 out, ldo, H, G, P, D, Dv, bs, window, keep, qb, epilogue, lam, eps, post, 1, 2,
-                nullptr, nullptr};
+                nullptr, nullptr, wmode, bias};
   if (is_bf16)
     hipLaunchKernelGGL((window_attn_kernel<bf16_t>), dim3(n_items), dim3(256), lds, st, a);
   else
@@ -352,7 +469,8 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
 // maps and mixes the rows of its own heads (buffers alternate between blocks).
 // Softmax weights stay fp32: P enters the second product as a bf16 high part plus a bf16
 // remainder, and the normaliser sums the fp32 weights.
-template <int HW, int P, bool TALK, bool SHARE, int ND, int NDV>
+// SIG: sigmoid weights (wmode 1) instead of the running softmax.
+template <int HW, int P, bool TALK, bool SHARE, int ND, int NDV, bool SIG = false>
 __global__ void __launch_bounds__(512)
 window_attn_mfma_kernel(const WinAttnArgs a) {
   constexpr int MW = HW * P;
@@ -416,11 +534,12 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
                                                         (d < D ? d : 0));
       qf[m][s] = d < D ? v : zero8;
     }
-  float mult[MW], slope[MW];
+  float mult[MW], slope[MW], sbias[MW];
 #pragma unroll
   for (int m = 0; m < MW; ++m) {
     mult[m] = a.mult[hs * P + m];
     slope[m] = a.slope ? a.slope[hs * P + m] : 0.f;
+    sbias[m] = (SIG && a.bias) ? a.bias[hs * P + m] : 0.f;
   }
   f32x4 acc[MW][NDV];
   float mrun[MW], lrun[MW];
@@ -573,6 +692,19 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
       float v[8];
+      if constexpr (SIG) {
+        // un-normalised sigmoid weights: no running maximum, nothing to rescale
+        alpha[m] = 1.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float z = (e < 4 ? sc[m][0][e] : sc[m][1][e - 4]) + sbias[m];
+          const float p = vis[e] ? 1.0f / (1.0f + exp2f(-z * LOG2E)) : 0.f;
+          const bf16_t hi = f2bf(p);
+          ph[m][e] = hi;
+          pl[m][e] = f2bf(p - bf2f(hi));
+        }
+        lrun[m] = 1.f;
+      } else {
       float mloc = -1e30f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
@@ -596,6 +728,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
       psum += __shfl_xor(psum, 32, 64);
       lrun[m] = lrun[m] * alpha[m] + psum;
       mrun[m] = mnew;
+      }
     }
     // O^T += V^T P^T: A rows = value columns 16 t + c, k = keys 8 g .. + 8 of the block
 #pragma unroll
@@ -604,7 +737,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 #pragma unroll
       for (int t = 0; t < NDV; ++t) {
         if (t < ndv) {
-          f32x4 o = acc[m][t] * alpha[m];
+          f32x4 o = SIG ? acc[m][t] : acc[m][t] * alpha[m];
           o = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][t], ph[m], o, 0, 0, 0);
           acc[m][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[j][t], pl[m], o, 0, 0, 0);
         }
@@ -695,8 +828,9 @@ window_attn_merge_kernel(const WinAttnArgs a) {
     const long pr = (row * M + h * P + pm) * NP;
     const float mz = lane < np ? a.part_ml[(pr + lane) * 2] : -1e30f;
     const float lz = lane < np ? a.part_ml[(pr + lane) * 2 + 1] : 0.f;
-    const float wz = __expf(mz - wave_max(mz));
-    const float inv = 1.0f / wave_sum(wz * lz);
+    // sigmoid weights: the partitions' sums simply add up
+    const float wz = a.wmode == 1 ? (lane < np ? 1.f : 0.f) : __expf(mz - wave_max(mz));
+    const float inv = a.wmode == 1 ? 1.f : 1.0f / wave_sum(wz * lz);
     float v0 = 0.f, v1 = 0.f;
 #pragma unroll 4
     for (int z = 0; z < np; ++z) {
@@ -751,13 +885,14 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
                                  const float* slope, const float* talk, const void* gate, long ldg,
                                  void* out, long ldo, int H, int G, int P, int D, int Dv, int bs,
                                  int window, int keep, int epilogue, const float* lam, float eps,
-                                 float post, int nparts, float* part_acc, float* part_ml,
-                                 hipStream_t st) {
+                                 float post, int wmode, const float* bias, int nparts,
+                                 float* part_acc, float* part_ml, hipStream_t st) {
   if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || bs < 1 || keep < 0 || !q ||
       !kc || !vc || !bt || !positions || !mult || !out)
     return EIA_BAD_SHAPE;
   if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
   if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam))) return EIA_BAD_SHAPE;
+  if ((wmode != 0 && wmode != 1) || (wmode == 1 && (talk || P != 1))) return EIA_BAD_SHAPE;
   if (!eia_window_attn_mfma_ok(H, G, P, D, Dv, bs, talk != nullptr)) return EIA_UNSUPPORTED;
   if (ldq % 8 || ldo % 4) return EIA_BAD_SHAPE;
   // key partitions: decode rows only (a row is its own work item), partials in the workspace
@@ -766,7 +901,7 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
                 out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post, nparts,
-                2, part_acc, part_ml};
+                2, part_acc, part_ml, wmode, bias};
   // raw-score buffers of the head-mixing form: two (one barrier per block) while they fit 48 KiB
   if (talk) a.raw_bufs = (size_t)2 * H * P * 128 * sizeof(f32x4) > 48 * 1024 ? 1 : 2;
   const int hw = wa_mfma_hw(H, P, talk != nullptr);
@@ -793,6 +928,9 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
     if (big) WA_LAUNCH1(HWV, PV, TK, SH, 4, 8);                                                 \
     else WA_LAUNCH1(HWV, PV, TK, SH, 2, 4);                                                     \
   } while (0)
+#define WA_LAUNCH_SIG(NDX, NDVX)                                                                \
+  hipLaunchKernelGGL((window_attn_mfma_kernel<1, 1, false, true, NDX, NDVX, true>), grid, block, \
+                     lds, st, a)
   // without head mixing the key width may be half the value width (a differential pair)
   const bool narrow_k = !talk && D <= 64 && Dv > 64;
   if (talk) {
@@ -802,10 +940,15 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
   } else if (P == 2) {
     if (narrow_k) WA_LAUNCH1(1, 2, false, true, 2, 8);
     else WA_LAUNCH(1, 2, false, true);
+  } else if (wmode == 1) {
+    if (narrow_k) WA_LAUNCH_SIG(2, 8);
+    else if (big) WA_LAUNCH_SIG(4, 8);
+    else WA_LAUNCH_SIG(2, 4);
   } else {
     if (narrow_k) WA_LAUNCH1(1, 1, false, true, 2, 8);
     else WA_LAUNCH(1, 1, false, true);
   }
+#undef WA_LAUNCH_SIG
 #undef WA_LAUNCH
 #undef WA_LAUNCH1
   if (nparts > 1)

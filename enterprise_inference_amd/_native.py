@@ -66,11 +66,11 @@ _SIGNATURES = {
     "eia_splitk_add_rmsnorm": [P, I, I, I, P, P, F, P, L, S],
     "eia_ln_residual": [P, L, P, P, P, L, F, I, I, I, S],
     "eia_ln_f32in": [P, L, P, P, L, F, I, I, I, S],
-    "eia_latent_prep": [P, L, I, I, P, P, L, I, I, P, I, I, I, P, IP, IP, P, L, F, I, I, S],
+    "eia_latent_prep": [P, L, I, I, P, P, L, I, I, P, I, I, I, P, IP, IP, P, L, F, I, F, I, I, S],
     "eia_latent_attn": [P, L, L, P, L, L, P, I, P, L, IP, I, IP, IP, IP, I, IP, P, L, P, L, L, F,
-                        I, I, I, I, I, I, S],
+                        I, I, I, I, I, I, P, I, F, I, S],
     "eia_latent_attn_mfma": [P, L, L, P, L, L, P, I, P, L, IP, I, IP, IP, IP, I, IP, P, L, P, L, L,
-                             F, I, I, I, I, I, I, P, P, S],
+                             F, I, I, I, I, I, I, P, I, F, I, P, P, S],
     "eia_token_shift_mix": [P, P, I, P, IP, IP, I, IP, P, L, I, I, I, S],
     "eia_wkv_scan": [P, P, P, P, L, P, L, P, P, P, P, P, P, I, IP, IP, IP, IP, P, L, F, I, I, I,
                      I, S],
@@ -82,9 +82,14 @@ _SIGNATURES = {
     "eia_qk_norm_cache": [P, L, P, I, P, I, I, I, I, I, I, I, I, I, P, P, P, L, P, P, P, L, IP, I, F,
                           I, I, S],
     "eia_window_attn": [P, L, P, P, IP, I, IP, IP, IP, IP, I, P, P, P, P, L, P, L, I, I, I, I, I,
-                        I, I, I, I, I, P, F, F, I, S],
+                        I, I, I, I, I, P, F, F, I, P, I, S],
     "eia_window_attn_mfma": [P, L, P, P, IP, I, IP, IP, IP, IP, I, P, P, P, P, L, P, L, I, I, I, I,
-                             I, I, I, I, I, P, F, F, I, P, P, S],
+                             I, I, I, I, I, P, F, F, I, P, I, P, P, S],
+    "eia_qk_rope_cache": [P, L, P, I, P, I, I, I, I, I, I, I, P, P, P, I, I, F, IP, P, L, P, P, IP,
+                          I, F, I, I, S],
+    "eia_add_rms": [P, L, P, I, P, P, L, P, I, P, P, P, P, L, F, I, I, I, S],
+    "eia_xielu": [P, L, P, I, P, P, L, I, I, I, S],
+    "eia_sigmoid_gate": [P, L, P, L, P, L, I, I, I, S],
     "eia_window_attn_mfma_ok": [I, I, I, I, I, I, I],
     "eia_ar_alloc": [P, L],
     "eia_moe_splitk_norm_route": [P, I, I, I, P, P, F, P, L, P, I, I, I, I, P, P, P, S],

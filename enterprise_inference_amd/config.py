@@ -139,11 +139,11 @@ class ModelConfig:
     def from_layer_list(cls, d: Dict[str, Any], name: str = "",
                         tensor_shapes: Optional[Dict[str, Any]] = None) -> "ModelConfig":
         """Designs whose config.json names the architecture in one string and lists the layers
-        one by one (Sekolorn, Vedadra): keys ``architecture``, ``vocab``, ``width``, ``norm.eps``
-        and ``layers`` (kept whole in ``extra["layers"]``); ``norm`` and an optional ``loop``
-        ({start, stop, times}: a run of layers repeated with the same weights) are kept whole
-        too.  Sizes the file leaves to the checkpoint (the rank of a wkv layer's decay branch)
-        come from ``tensor_shapes`` when given."""
+        one by one (Sekolorn, Vedadra, Gapidra): keys ``architecture``, ``vocab``, ``width``,
+        ``norm.eps`` and ``layers`` (kept whole in ``extra["layers"]``); ``norm``, ``embedding``
+        ({scale}) and an optional ``loop`` ({start, stop, times}: a run of layers repeated with
+        the same weights) are kept whole too.  Sizes the file leaves to the checkpoint (the rank
+        of a wkv layer's decay branch) come from ``tensor_shapes`` when given."""
         import copy
         layers = copy.deepcopy(d["layers"])
         for i, L in enumerate(layers):
@@ -160,6 +160,7 @@ class ModelConfig:
                    max_position_embeddings=1 << 20,      # the design sets no limit
                    rms_norm_eps=eps, layer_norm_eps=eps,
                    name=name, extra={"layers": layers, "norm": dict(d.get("norm") or {}),
+                                     "embedding": dict(d.get("embedding") or {}),
                                      "loop": dict(d["loop"]) if d.get("loop") else None})
 
     @classmethod

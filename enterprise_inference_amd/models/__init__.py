@@ -19,6 +19,7 @@ _REGISTRY: Dict[str, str] = {
     "OPTForCausalLM": "opt:OPTForCausalLM",
     "Sekolorn": "sekolorn:SekolornForCausalLM",
     "Vedadra": "vedadra:VedadraForCausalLM",
+    "Gapidra": "gapidra:GapidraForCausalLM",
     "BertModel": "bert:BertEmbeddingModel",
     "XLMRobertaModel": "bert:BertEmbeddingModel",
     "XLMRobertaForSequenceClassification": "bert:CrossEncoderModel",

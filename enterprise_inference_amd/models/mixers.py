@@ -6,7 +6,10 @@ returns the mixer output in the activation dtype.
 * ``LatentAttentionMixer`` -- attention through low-rank latents: queries and keys/values are
   up-projected from RMS-normed latents, a rotated key part is shared by all heads, and only the
   KV latent and that key part are cached (one row per token, shared by every head; a layer may
-  read another layer's rows).  Runs in the absorbed form (ops/latent_attention.py).
+  read another layer's rows).  Runs in the absorbed form (ops/latent_attention.py).  Options:
+  queries straight from the layer input (``q_rank`` 0), a sliding window, a per-head sink in
+  the softmax denominator, either pair layout of the rotation, and an output gate per head or
+  per element.
 * ``WKVMixer`` -- token-shift mixing and a per-head matrix-state recurrence with data-dependent
   per-channel decay on per-sequence state slots (ops/wkv.py).
 * ``TalkingWindowAttentionMixer`` -- sliding-window softmax attention without rotation: RMS-normed
@@ -14,7 +17,10 @@ returns the mixer output in the activation dtype.
   penalty, mixing of the heads' scores before the softmax and a sigmoid output gate.
 * ``DifferentialAttentionMixer`` -- two softmax maps per head over the same values, combined as
   ``a1 - lambda * a2`` and RMS-normed per head; sliding window plus always-visible first tokens.
-  Both run on token-major paged K / V rows (``PagedKVRows``, ops/window_attention.py).
+* ``SigmoidWindowAttentionMixer`` -- grouped-query sliding-window attention whose weights are
+  ``sigmoid(score + bias_h)``, not normalised over the keys; queries and keys are RMS-normed as
+  whole projections and then rotated.
+  All three run on token-major paged K / V rows (``PagedKVRows``, ops/window_attention.py).
 """
 
 from __future__ import annotations
@@ -22,8 +28,10 @@ from __future__ import annotations
 import torch
 import torch.nn as nn
 
+from ..ops import activation as act_ops
 from ..ops import gemm
 from ..ops import latent_attention as lat_ops
+from ..ops import rotary as rot_ops
 from ..ops import window_attention as win_ops
 from ..ops import wkv as wkv_ops
 from ..ops.attention import AttentionMetadata
@@ -58,59 +66,99 @@ class RecurrentState:
 
 
 class LatentAttentionMixer(nn.Module):
+    """Keys and values of every head are up-projections (``uk``, ``uv``) of one RMS-normed
+    latent per token; a rotated key part is shared by the heads; only both are cached.
+
+    ``q_rank`` > 0: queries are up-projected (``uq``) from an RMS-normed query latent; 0: they
+    come straight from the layer input (``q`` rows in the fused projection).  ``gate``: "head"
+    (one sigmoid per head, applied to the attended latent), "element" (sigmoid(W_g x) on the
+    concatenated heads, after the value up-projection) or None.  ``window`` > 0: sliding window.
+    ``sink``: a learned per-head term exp(sink_h) in the softmax denominator.  ``rot_half``:
+    rotation pairs (i, i + dims/2) instead of (2i, 2i+1); ``rot_scaling``: frequency
+    interpolation (ops/rotary.py rotary_frequencies).  ``defer_out``: hand the output
+    projection's split-K partials to the caller's boundary step."""
+
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
                  q_rank: int, scale: float, rot_dims: int, rot_base: float, eps: float,
-                 own_kv: bool, dtype, device):
+                 own_kv: bool, dtype, device, *, gate: str = "head", window: int = 0,
+                 sink: bool = False, rot_half: bool = False, rot_scaling=None,
+                 defer_out: bool = False):
         super().__init__()
         if pstate.tp_size() != 1:
             raise NotImplementedError("latent attention runs on one rank (no head sharding yet)")
+        if gate not in ("head", "element", None):
+            raise ValueError(f"latent attention gate {gate!r}")
+        if rot_dims > rot_dim or rot_dims % 2:
+            raise ValueError("rot.dims must be even and at most rot_dim")
         self.width, self.heads, self.dim, self.rot_dim, self.vdim = width, heads, dim, rot_dim, vdim
         self.kv_rank, self.q_rank, self.scale, self.eps = kv_rank, q_rank, float(scale), float(eps)
         self.rot_dims = rot_dims
         self.own_kv = own_kv
-        # one fused down-projection of the layer input: [query latent | KV latent | shared rotary
-        # key | head gates]; a layer reading another layer's cache has no KV rows
+        self.gate, self.window, self.rot_half, self.defer_out = gate, int(window), rot_half, defer_out
+        # one fused projection of the layer input: [query latent or queries | KV latent | shared
+        # rotary key | gates]; a layer reading another layer's cache has no KV rows
         self.kv_rows = kv_rank + rot_dim if own_kv else 0
+        self.q_rows = q_rank if q_rank else heads * (dim + rot_dim)
+        self.gate_rows = {"head": heads, "element": heads * vdim, None: 0}[gate]
         # (rows padded with zeros to a multiple of 64: decode-sized batches then run the
         # weight-streaming GEMM, whose row tiles need it; the pad columns are never read)
-        n = q_rank + self.kv_rows + heads
+        n = self.q_rows + self.kv_rows + self.gate_rows
         self.down = _param((-(-n // 64) * 64, width), dtype, device)
         self.down.data[n:].zero_()
         self.down.weight_loader = self._load_down
-        self.q_norm = _plain((q_rank,), dtype, device)
+        self.q_norm = _plain((q_rank,), dtype, device) if q_rank else None
         self.kv_norm = _plain((kv_rank,), dtype, device) if own_kv else None
-        self.uq = _plain((heads * (dim + rot_dim), q_rank), dtype, device)
+        self.uq = _plain((heads * (dim + rot_dim), q_rank), dtype, device) if q_rank else None
         self.uk = _plain((heads * dim, kv_rank), dtype, device)
         self.uv = _plain((heads * vdim, kv_rank), dtype, device)
         self.o = _plain((width, heads * vdim), dtype, device)
-        self.inv_freq = lat_ops.inv_frequencies(rot_dims, rot_base, device)
+        self.sink = _plain((heads,), dtype, device) if sink else None
+        # fp32 copy of the sinks for the attention launch, refreshed IN PLACE after a weight
+        # load (captured decode graphs hold its address)
+        self.sink_f32 = torch.zeros(heads, dtype=torch.float32, device=device) if sink else None
+        self.inv_freq, self.rot_amp = rot_ops.rotary_frequencies(rot_dims, rot_base, rot_scaling,
+                                                                 device)
         self.qblock = lat_ops.query_block(heads, kv_rank, rot_dim,
                                           dtype if torch.device(device).type == "cuda"
                                           else torch.float32)
 
-    def _load_down(self, param, loaded, shard_id=None):
-        off = {"dq": 0, "dkv": self.q_rank, "g": self.q_rank + self.kv_rows}[shard_id]
-        if param.data[off:off + loaded.shape[0]].shape != loaded.shape:
-            raise ValueError(f"latent attention {shard_id}: shape {tuple(loaded.shape)}")
-        param.data[off:off + loaded.shape[0]].copy_(loaded)
+    def refresh(self) -> None:
+        if self.sink is not None:
+            self.sink_f32.copy_(self.sink.float())
 
-    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: LatentKVCache) -> torch.Tensor:
+    def _load_down(self, param, loaded, shard_id=None):
+        off = {"dq": 0, "q": 0, "dkv": self.q_rows, "g": self.q_rows + self.kv_rows}[shard_id]
+        rows = {"dq": self.q_rows, "q": self.q_rows, "dkv": self.kv_rows, "g": self.gate_rows}[shard_id]
+        if loaded.shape[0] != rows or param.data[off:off + rows].shape != loaded.shape:
+            raise ValueError(f"latent attention {shard_id}: shape {tuple(loaded.shape)}")
+        param.data[off:off + rows].copy_(loaded)
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: LatentKVCache):
         T = xb.shape[0]
         H, D, rd, R = self.heads, self.dim, self.rot_dim, self.kv_rank
         fused = gemm.linear(xb, self.down)
-        cq = lat_ops.latent_prep(fused, 0, self.q_rank, self.q_norm, self.q_rank, R, self.kv_norm,
-                                 self.q_rank + R, rd, self.rot_dims, self.inv_freq, md.positions,
-                                 md.slot_mapping, cache.rows if self.own_kv else None, self.eps)
-        q = gemm.linear(cq, self.uq).view(T, H, D + rd)
+        cq = lat_ops.latent_prep(fused, 0, self.q_rank, self.q_norm, self.q_rows, R, self.kv_norm,
+                                 self.q_rows + R, rd, self.rot_dims, self.inv_freq, md.positions,
+                                 md.slot_mapping, cache.rows if self.own_kv else None, self.eps,
+                                 self.rot_half, self.rot_amp)
+        if self.q_rank:
+            q = gemm.linear(cq, self.uq).view(T, H, D + rd)
+        else:
+            q = fused[:, :self.q_rows].view(T, H, D + rd)
         # key up-projection folded into the query: q_abs[t, h] = W_uk[h]^T q_nope[t, h]
         q_abs = torch.bmm(q[:, :, :D].transpose(0, 1), self.uk.view(H, D, R)).transpose(0, 1)
-        g0 = self.q_rank + self.kv_rows
-        gate = fused[:, g0:g0 + H]
+        g0 = self.q_rows + self.kv_rows
         lat = lat_ops.latent_attention(q_abs, q[:, :, D:], self.inv_freq, self.rot_dims,
-                                       cache.rows, md, gate, self.scale)
+                                       cache.rows, md,
+                                       fused[:, g0:g0 + H] if self.gate == "head" else None,
+                                       self.scale, self.window, self.sink_f32, self.rot_half,
+                                       self.rot_amp)
         # value up-projection of the attended latent, heads concatenated
         o = torch.bmm(lat.transpose(0, 1), self.uv.view(H, self.vdim, R).transpose(1, 2))
-        return gemm.linear(o.transpose(0, 1).reshape(T, H * self.vdim), self.o)
+        o = o.transpose(0, 1).reshape(T, H * self.vdim)
+        if self.gate == "element":
+            o = act_ops.sigmoid_gate(o, fused[:, g0:g0 + self.gate_rows])
+        return gemm.linear(o, self.o, defer_reduce=self.defer_out)
 
 
 class WKVMixer(nn.Module):
@@ -197,7 +245,7 @@ class _WindowMixerBase(nn.Module):
     maps = 1
 
     def _setup(self, width, heads, kv_heads, dim, vdim, scale, window, keep, eps, parts, bias,
-               dtype, device):
+               dtype, device, norm_sizes=None):
         if pstate.tp_size() != 1:
             raise NotImplementedError("window attention mixers run on one rank (no head sharding yet)")
         if heads % kv_heads:
@@ -216,8 +264,10 @@ class _WindowMixerBase(nn.Module):
             self.proj_bias = _param((_pad64(n),), dtype, device)
             self.proj_bias.data.zero_()
             self.proj_bias.weight_loader = self._load_part
-        self.q_norm = _plain((dim,), dtype, device)
-        self.k_norm = _plain((dim,), dtype, device)
+        # norm weights: one per map entry (shared by the maps), or ``norm_sizes`` = (query, key)
+        qn, kn = norm_sizes or (dim, dim)
+        self.q_norm = _plain((qn,), dtype, device)
+        self.k_norm = _plain((kn,), dtype, device)
         self.o = _plain((width, heads * vdim), dtype, device)
         M = heads * self.maps
         # fp32 constants of the attention launch, refreshed IN PLACE after a weight load
@@ -317,3 +367,42 @@ class DifferentialAttentionMixer(_WindowMixerBase):
 
     def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows) -> torch.Tensor:
         return gemm.linear(self._attend(xb, md, cache, "v"), self.o, defer_reduce=True)
+
+
+class SigmoidWindowAttentionMixer(_WindowMixerBase):
+    """Grouped-query sliding-window attention with un-normalised weights: a visible key j weighs
+    sigmoid((q_h . k_j) scale + pb_h) for head h; out_h = sum_j weight_j v_j.  The query and the
+    key projection are each RMS-normed as ONE vector (weights of their full size) before the
+    first ``rot_dims`` entries of every head turn by the position (pairs (2i, 2i+1), or
+    (i, i + rot_dims/2) with ``rot_half``; ``rot_scaling`` as in ops/rotary.py
+    rotary_frequencies).  No biases, no gate."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 window: int, rot_dims: int, rot_base: float, rot_scaling, eps: float, dtype,
+                 device, rot_half: bool = False):
+        super().__init__()
+        if rot_dims > dim or rot_dims % 2:
+            raise ValueError("rot.dims must be even and at most dim")
+        self._setup(width, heads, kv_heads, dim, vdim, scale, window, 0, eps,
+                    [("q", heads * dim), ("k", kv_heads * dim), ("v", kv_heads * vdim)], False,
+                    dtype, device, norm_sizes=(heads * dim, kv_heads * dim))
+        self.rot_dims, self.rot_half = int(rot_dims), rot_half
+        self.inv_freq, self.rot_amp = rot_ops.rotary_frequencies(rot_dims, rot_base, rot_scaling,
+                                                                 device)
+        self.pb = _plain((heads,), dtype, device)
+        self.spec.weights = 1
+        self.spec.bias = torch.zeros(heads, dtype=torch.float32, device=device)
+
+    def refresh(self) -> None:
+        self.spec.bias.copy_(self.pb.float())
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows):
+        fused = gemm.linear(xb, self.proj, None, defer_reduce=True)
+        q = win_ops.qk_rope_cache(fused, self.offsets["q"][0], self.offsets["k"][0],
+                                  self.offsets["v"][0], self.heads, self.kv_heads, self.dim,
+                                  self.kv_heads * self.vdim, self.q_norm, self.k_norm,
+                                  self.inv_freq, self.rot_dims, self.rot_half, self.rot_amp,
+                                  md.positions, cache.k, cache.v, md.slot_mapping, self.eps)
+        a = win_ops.window_attention(q, cache.k, cache.v, md, self.spec, None)
+        # may return gemm.SplitK: the layer's boundary step reduces it
+        return gemm.linear(a, self.o, defer_reduce=True)

@@ -198,16 +198,30 @@ class MixtralMoE(nn.Module):
 
 
 class UngatedMLP(nn.Module):
-    """W_down act(W_up x) without a gate branch (act: squared ReLU)."""
+    """W_down act(W_up x) without a gate branch.  ``act``: "relu2" (squared ReLU) or "xielu"
+    (softplus(p) z^2 + z/2 above zero, (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 below, with
+    the layer's two learned numbers (p, q) in the parameter ``act``).  With ``defer`` the
+    decode-sized products hand their split-K partial sums on: the up-projection's to the
+    activation kernel, the down-projection's to the caller's boundary step."""
 
-    def __init__(self, hidden: int, inter: int, dtype, device):
+    def __init__(self, hidden: int, inter: int, dtype, device, act: str = "relu2",
+                 defer: bool = False):
         super().__init__()
+        if act not in ("relu2", "xielu"):
+            raise ValueError(f"UngatedMLP: unknown activation {act!r}")
         self.up = ReplicatedLinear(hidden, inter, dtype=dtype, device=device)
         self.down = ReplicatedLinear(inter, hidden, dtype=dtype, device=device)
+        self.kind, self.defer = act, defer
+        if act == "xielu":
+            self.act = _param((2,), dtype, device)
+            self.act.weight_loader = lambda p, t, sid=None: p.data.copy_(t.reshape(2))
 
     def forward(self, x):
-        from ..ops import activation
-        return self.down(activation.relu2(self.up(x)))
+        from ..ops import activation, gemm
+        if self.kind == "relu2":
+            return self.down(activation.relu2(self.up(x)))
+        z = activation.xielu(gemm.linear(x, self.up.weight, defer_reduce=self.defer), self.act)
+        return gemm.linear(z, self.down.weight, defer_reduce=self.defer)
 
 
 class GroupRoutedMoE(nn.Module):

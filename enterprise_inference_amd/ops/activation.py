@@ -5,7 +5,7 @@ from __future__ import annotations
 import torch
 
 from . import reference as ref
-from ._dispatch import check, lib, ptr, stream, use_hip
+from ._dispatch import check, lib, ptr, require, stream, use_hip
 
 _KIND = {"silu": 0, "swiglu": 0, "gelu_tanh": 1, "gelu_pytorch_tanh": 1, "gelu_new": 1,
          "gelu": 2, "gelu_erf": 2}
@@ -62,4 +62,55 @@ def relu2(x: torch.Tensor) -> torch.Tensor:
     out = torch.empty_like(x)
     check(lib().eia_relu2(ptr(out), ptr(x), x.numel(), 1 if x.dtype == torch.bfloat16 else 0,
                           stream(x)), "relu2")
+    return out
+
+
+def xielu(x, pq: torch.Tensor) -> torch.Tensor:
+    """xIELU with the two learned numbers ``pq`` = (p, q) read from device memory:
+    z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2, evaluated
+    in fp32.  x [T, F] in the activation dtype, or a ``gemm.SplitK`` (fp32 partial sums of the
+    up-projection, summed here) -> [T, F] in pq's dtype."""
+    from .gemm import SplitK
+    split = isinstance(x, SplitK)
+    if split and not (x.part.is_cuda and x.bias is None and x.N % 4 == 0 and x.part.is_contiguous()):
+        x = x.materialize() if x.part.is_cuda else (x.part.sum(0) + (
+            x.bias.float() if x.bias is not None else 0.0)).to(pq.dtype)
+        split = False
+    if not split and not use_hip(x):
+        z = x.float()
+        ap = torch.nn.functional.softplus(pq[0].float())
+        aq = 0.5 + torch.nn.functional.softplus(pq[1].float())
+        pos = ap * z * z + 0.5 * z
+        neg = aq * (torch.expm1(torch.clamp(z, max=0.0)) - z) + 0.5 * z
+        return torch.where(z > 0, pos, neg).to(x.dtype)
+    dt = pq.dtype
+    require(dt in (torch.bfloat16, torch.float32) and pq.numel() == 2 and pq.is_contiguous(),
+            "xielu: two numbers, bf16 or fp32")
+    if split:
+        T, F = x.M, x.N
+        out = torch.empty(T, F, dtype=dt, device=pq.device)
+        check(lib().eia_xielu(None, 0, ptr(x.part), x.sk, ptr(pq), ptr(out), out.stride(0), T, F,
+                              1 if dt == torch.bfloat16 else 0, stream(out)), "xielu")
+        return out
+    require(x.dim() == 2 and x.stride(1) == 1 and x.dtype == dt, "xielu: row layout")
+    T, F = x.shape
+    out = torch.empty(T, F, dtype=dt, device=x.device)
+    check(lib().eia_xielu(ptr(x), x.stride(0), None, 0, ptr(pq), ptr(out), out.stride(0), T, F,
+                          1 if dt == torch.bfloat16 else 0, stream(out)), "xielu")
+    return out
+
+
+def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
+    """a * sigmoid(gate), element by element (fp32 inside); a, gate [T, N] rows with a contiguous
+    last dim (either may be a column slice of a wider row) -> [T, N] contiguous."""
+    if not use_hip(a, gate):
+        return (a.float() * torch.sigmoid(gate.float())).to(a.dtype)
+    require(a.dim() == 2 and a.shape == gate.shape and a.stride(1) == 1 and gate.stride(1) == 1
+            and a.dtype == gate.dtype and a.dtype in (torch.bfloat16, torch.float32),
+            "sigmoid_gate: layout")
+    T, N = a.shape
+    out = torch.empty(T, N, dtype=a.dtype, device=a.device)
+    check(lib().eia_sigmoid_gate(ptr(a), a.stride(0), ptr(gate), gate.stride(0), ptr(out),
+                                 out.stride(0), T, N, 1 if a.dtype == torch.bfloat16 else 0,
+                                 stream(a)), "sigmoid_gate")
     return out

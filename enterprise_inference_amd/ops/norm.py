@@ -170,3 +170,63 @@ def group_norm_step(x: torch.Tensor, groups: int, eps: float, y=None,
                           ptr(ybias), ptr(w_post), ptr(x), ptr(add), ptr(w_next), ptr(h), W,
                           float(eps), T, W, groups, 1 if bf else 0, stream(x)), "gnorm")
     return h
+
+
+def residual_rms_step(x: torch.Tensor, eps: float, ys=(), w_next: Optional[torch.Tensor] = None
+                      ) -> Optional[torch.Tensor]:
+    """Boundary of a layer whose sublayers run side by side on one normed input, around an fp32
+    residual stream x [T, W], in one pass over the row:
+
+        x += y            for every y in ``ys`` (at most two sublayer outputs, un-normed, in place)
+        h  = x / sqrt(mean(x^2) + eps) * w_next      (w_next given: returned in its dtype)
+
+    All arithmetic is fp32.  A y is a tensor in the activation dtype or a ``gemm.SplitK`` (the
+    fp32 partial sums of the GEMM that produced it, plus its bias), reduced here."""
+    from .gemm import SplitK
+    T, W = x.shape
+    ys = [y for y in ys if y is not None]
+    require(len(ys) <= 2, "residual_rms_step: at most two sublayer outputs")
+
+    def dense(y):
+        if isinstance(y, SplitK):
+            return y.part.sum(0) + (y.bias.float() if y.bias is not None else 0.0)
+        return y.float()
+
+    if use_hip(x) and W % 4:
+        # the kernel sums partials in 16-byte units; no GEMM of the framework produces other widths
+        ys = [dense(y) if isinstance(y, SplitK) else y for y in ys]
+    if not use_hip(x):
+        for y in ys:
+            x += dense(y)
+        if w_next is None:
+            return None
+        return (x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w_next.float()).to(w_next.dtype)
+    require(x.dtype == torch.float32 and x.is_contiguous(), "residual_rms_step: fp32 stream")
+    dt = w_next.dtype if w_next is not None else None
+    args = []
+    for y in ys:
+        if isinstance(y, SplitK):
+            require(y.M == T and y.N == W and y.part.is_contiguous() and
+                    y.part.dtype == torch.float32, "residual_rms_step: partials")
+            dt = dt or (y.bias.dtype if y.bias is not None else None)
+            args.append((None, 0, y.part, y.sk, y.bias))
+        else:
+            require(y.shape == x.shape and y.stride(-1) == 1, "residual_rms_step: y layout")
+            dt = dt or y.dtype
+            require(y.dtype == dt, "residual_rms_step: one activation dtype")
+            args.append((y, y.stride(0), None, 0, None))
+    for a in args:
+        require(a[4] is None or a[4].dtype == dt, "residual_rms_step: bias dtype")
+    dt = dt or torch.float32
+    require(dt in (torch.bfloat16, torch.float32), "residual_rms_step: bf16 or fp32")
+    while len(args) < 2:
+        args.append((None, 0, None, 0, None))
+    h = None
+    if w_next is not None:
+        require(w_next.numel() == W, "residual_rms_step: weight size")
+        h = torch.empty(T, W, dtype=w_next.dtype, device=x.device)
+    (y1, l1, p1, s1, b1), (y2, l2, p2, s2, b2) = args
+    check(lib().eia_add_rms(ptr(y1), l1, ptr(p1), s1, ptr(b1), ptr(y2), l2, ptr(p2), s2, ptr(b2),
+                            ptr(x), ptr(w_next), ptr(h), W, float(eps), T, W,
+                            1 if dt == torch.bfloat16 else 0, stream(x)), "add_rms")
+    return h

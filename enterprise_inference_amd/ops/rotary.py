@@ -67,3 +67,28 @@ def rope_qkv_cache(qkv, positions: Optional[torch.Tensor],
         num_heads, num_kv_heads, head_dim, k_cache.shape[2],
         1 if (rotary is None or rotary.is_neox) else 0, stream(q)), "rope_qkv_cache")
     return q
+
+
+def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None, device=None):
+    """(f [dims/2] fp32, amp): the angle of pair i at position p is p * f_i, and cos and sin are
+    multiplied by amp.  f_i = base^(-2i/dims); with ``scaling`` = {factor, original, fast, slow}
+    (YaRN) the pairs that turn fewer than ``slow`` times over ``original`` positions are slowed
+    by ``factor``, those that turn more than ``fast`` times keep their frequency, the ones
+    between are blended linearly in the pair index, and amp = 0.1 ln(factor) + 1.  Evaluated in
+    float64 and rounded once."""
+    import math
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(dims, 1))
+    amp = 1.0
+    if scaling:
+        factor, orig = float(scaling["factor"]), float(scaling["original"])
+
+        def pair_of(turns: float) -> float:       # the (real-valued) pair index turning that often
+            return dims * math.log(orig / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))
+
+        lo = max(math.floor(pair_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(scaling["slow"]))), dims - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        amp = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32).to(device), float(amp)

@@ -7,7 +7,8 @@ keys of a value column are one 16-byte load).  A query row carries
 map ``h*P + c`` reads key map ``(h // (H//G))*P + c`` and value head ``h // (H//G)``.  Per map
 the score of (query position i, key j) is ``(q.k) * mult[m] - slope[m]*(i-j)``, optionally mixed
 across maps by a matrix (``talk``), masked to ``j <= i and (i-j < window or j < keep)`` and
-soft-maxed.  ``spec.epilogue`` 0 multiplies the heads by ``sigmoid(gate)``; 1 combines a head's
+soft-maxed -- or, with ``spec.weights`` 1, every visible key simply weighs
+``sigmoid(score + bias[m])`` and nothing is normalised over the keys.  ``spec.epilogue`` 0 multiplies the heads by ``sigmoid(gate)``; 1 combines a head's
 two maps as ``a1 - lam*a2``, divides by the root mean square over the head and scales.
 
 A step's rows are [decode rows (1 per sequence) | prefill chunks]; both parts read the cache
@@ -46,6 +47,8 @@ class WindowSpec:
     lam: Optional[torch.Tensor] = None      # [1], the differential weight (epilogue 1)
     eps: float = 0.0
     post: float = 1.0
+    weights: int = 0                # 0: softmax over the visible keys; 1: sigmoid(score + bias)
+    bias: Optional[torch.Tensor] = None     # [H*P], added to the score inside the sigmoid
 
 
 def build_work(q_lens: List[int], qblock: int) -> List[int]:
@@ -166,6 +169,79 @@ def qk_norm_cache(fused, q_off: int, k_off: int, v_off: int, mq: int, mk: int,
     return q, gate
 
 
+def qk_rope_cache(fused, q_off: int, k_off: int, v_off: int, mq: int, mk: int, dim: int,
+                  v_width: int, q_w: torch.Tensor, k_w: torch.Tensor, inv_freq: torch.Tensor,
+                  rot_dims: int, rot_half: bool, rot_amp: float, positions: torch.Tensor,
+                  k_cache: torch.Tensor, v_cache: torch.Tensor, slot_mapping: torch.Tensor,
+                  eps: float) -> torch.Tensor:
+    """One pass over fused projection rows [T, *] for heads that are normed as ONE vector and
+    then rotated: the ``mq * dim`` query columns at ``q_off`` are divided by their common root
+    mean square and multiplied by ``q_w`` [mq*dim] (``q_w`` None: no norm), then the first
+    ``rot_dims`` entries of every head turn by the token's position (pairs (2i, 2i+1), or
+    (i, i + rot_dims/2) with ``rot_half``; angle position * inv_freq[i]; cos and sin times
+    ``rot_amp``) and the row is returned [T, mq*dim]; the ``mk * dim`` key columns at ``k_off``
+    get the same with ``k_w`` and land in the token's key row, the ``v_width`` value columns at
+    ``v_off`` in its value columns.  Rows with a slot < 0 write no cache.  ``fused`` may be a
+    ``gemm.SplitK`` (fp32 partial sums of the projection, summed here)."""
+    from .gemm import SplitK
+    from .latent_attention import _rotate_pairs
+    split = isinstance(fused, SplitK)
+    if split and (not fused.part.is_cuda or fused.N % 4):
+        fused = fused.part.sum(0) + (fused.bias.float() if fused.bias is not None else 0.0)
+        fused = fused if not fused.is_cuda else fused.to(k_cache.dtype)
+        split = False
+    if not split and not use_hip(fused):
+        T = fused.shape[0]
+        f = fused.float()
+
+        def side(off, m, w):
+            x = f[:, off:off + m * dim]
+            if w is not None:
+                x = _rms(x, eps) * w.float()
+            x = _rotate_pairs(x.reshape(T, m, dim), positions[:T, None], inv_freq, rot_dims,
+                              rot_half, rot_amp)
+            return x.reshape(T, m * dim)
+
+        q, k = side(q_off, mq, q_w), side(k_off, mk, k_w)
+        sm = slot_mapping[:T].long()
+        ok = sm >= 0
+        k_cache.view(-1, k_cache.shape[-1])[sm[ok]] = k[ok].to(k_cache.dtype)
+        bs = v_cache.shape[2]
+        v_cache[sm[ok] // bs, :, sm[ok] % bs] = f[:, v_off:v_off + v_width][ok].to(v_cache.dtype)
+        return q.to(k_cache.dtype)
+    dt = k_cache.dtype
+    bf = dt == torch.bfloat16
+    require(bf or dt == torch.float32, "qk_rope_cache: bf16 or fp32")
+    if split:
+        T, width = fused.M, fused.N
+        require(fused.part.dtype == torch.float32 and fused.part.is_contiguous() and
+                (fused.bias is None or fused.bias.dtype == dt), "qk_rope_cache: partials")
+    else:
+        T, width = fused.shape
+        require(fused.stride(1) == 1 and fused.dtype == dt, "qk_rope_cache: fused row layout")
+    require(max(q_off + mq * dim, k_off + mk * dim, v_off + v_width) <= width,
+            "qk_rope_cache: columns outside the row")
+    require(v_cache.dtype == dt and k_cache.is_contiguous() and v_cache.is_contiguous() and
+            k_cache.shape[-1] == mk * dim and v_cache.shape[1] == v_width and
+            v_cache.shape[2] == k_cache.shape[1], "qk_rope_cache: cache layout")
+    require((q_w is None or (q_w.dtype == dt and q_w.numel() == mq * dim)) and
+            (k_w is None or (k_w.dtype == dt and k_w.numel() == mk * dim)),
+            "qk_rope_cache: norm weights")
+    require(0 <= rot_dims <= dim and rot_dims % 2 == 0 and inv_freq.dtype == torch.float32 and
+            inv_freq.numel() >= rot_dims // 2, "qk_rope_cache: rotation")
+    require(slot_mapping.dtype == torch.int32 and slot_mapping.numel() >= T and
+            positions.dtype == torch.int32 and positions.numel() >= T, "int32 slots and positions")
+    q = torch.empty(T, mq * dim, dtype=dt, device=k_cache.device)
+    check(lib().eia_qk_rope_cache(
+        None if split else ptr(fused), width if split else fused.stride(0),
+        ptr(fused.part) if split else None, fused.sk if split else 0,
+        ptr(fused.bias) if split else None, q_off, k_off, v_off, mq, mk, dim, v_width, ptr(q_w),
+        ptr(k_w), ptr(inv_freq), rot_dims, 1 if rot_half else 0, float(rot_amp), ptr(positions),
+        ptr(q), q.stride(0), ptr(k_cache), ptr(v_cache), ptr(slot_mapping), k_cache.shape[1],
+        float(eps), T, 1 if bf else 0, stream(q)), "qk_rope_cache")
+    return q
+
+
 def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpec, seq_of_row):
     """Plain per-row attention over the paged rows (CPU path)."""
     H, G, P, D, Dv = spec.heads, spec.kv_heads, spec.maps, spec.dim, spec.vdim
@@ -186,7 +262,11 @@ def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpe
             sc = sc - spec.slope[:, None] * (i - js).float()[None, :]
         if spec.talk is not None:
             sc = spec.talk @ sc
-        w = torch.softmax(sc, -1).view(H, P, len(js))
+        if spec.weights == 1:
+            w = torch.sigmoid(sc + (spec.bias[:, None] if spec.bias is not None else 0.0))
+        else:
+            w = torch.softmax(sc, -1)
+        w = w.view(H, P, len(js))
         a = torch.einsum("hpn,nhd->hpd", w, vals)
         if spec.epilogue == 0:
             o = a[:, 0].reshape(H * Dv)
@@ -229,7 +309,9 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     require(gate is None or (gate.dtype == q.dtype and gate.stride(1) == 1 and
                              gate.shape[1] >= H * Dv), "window_attention: gate layout")
     require(md.positions.dtype == torch.int32, "positions int32")
-    for t in (spec.mult, spec.slope, spec.talk, spec.lam):
+    require(spec.weights in (0, 1) and (spec.weights == 0 or (spec.talk is None and P == 1)),
+            "window_attention: sigmoid weights come without head mixing or map pairs")
+    for t in (spec.mult, spec.slope, spec.talk, spec.lam, spec.bias):
         require(t is None or (t.dtype == torch.float32 and t.is_cuda and t.is_contiguous()),
                 "window_attention: fp32 device constants")
     bs = k_cache.shape[1]
@@ -253,16 +335,16 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                 ptr(md.positions[lo:]), ptr(cu), ptr(work), ptr(lens), n_items, ptr(spec.mult),
                 ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0,
                 ptr(o), o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep,
-                spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), NP, ptr(pa),
-                ptr(pm), stream(q)), "window_attn_mfma")
+                spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), spec.weights,
+                ptr(spec.bias), NP, ptr(pa), ptr(pm), stream(q)), "window_attn_mfma")
             return
         check(lib().eia_window_attn(
             ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),
             ptr(md.positions[lo:]), ptr(cu), ptr(work), ptr(lens), n_items, ptr(spec.mult),
             ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0, ptr(o),
             o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep, qb,
-            spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), 1 if bf else 0,
-            stream(q)), "window_attn")
+            spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), spec.weights,
+            ptr(spec.bias), 1 if bf else 0, stream(q)), "window_attn")
 
     if nd:
         launch(0, nd, md.decode_block_tables, md.decode_seq_lens, None, None, 1)
