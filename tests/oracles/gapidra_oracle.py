@@ -83,9 +83,27 @@ def visible(i, window):
     return range(lo, i + 1)
 
 
+def latent_core(q_plain, q_rot, lat, krot, uk, uv, i, window, scale, sink):
+    """Heads [H, Dv] of position i.  q_plain [H, D], q_rot [H, rd] (already rotated); lat[j] the
+    normed latent and krot[j] the rotated shared key part of position j; uk [H, D, R], uv
+    [H, Dv, R]; sink [H]: one more term exp(sink_h) in head h's denominator."""
+    H, Dv = uv.shape[0], uv.shape[1]
+    heads = np.zeros((H, Dv))
+    js = list(visible(i, window))
+    for a in range(H):
+        sc = np.array([(q_plain[a] @ (uk[a] @ lat[j]) + q_rot[a] @ krot[j]) * scale for j in js])
+        top = max(sc.max(), float(sink[a]))
+        e = np.exp(sc - top)
+        den = e.sum() + math.exp(float(sink[a]) - top)
+        for wgt, j in zip(e / den, js):
+            heads[a] += wgt * (uv[a] @ lat[j])
+    return heads
+
+
 def latent_attention(hs, W, pre, m, eps):
     """hs: list of mixer inputs (one per position) -> list of mixer outputs."""
-    H, D, rd, Dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+    H, D, rd, R = m["heads"], m["dim"], m["rot_dim"], m["kv_rank"]
+    Dv = m.get("vdim", D)
     rot = m.get("rot") or {"dims": rd, "base": 10000.0}
     freqs, amp = frequencies(rot)
     window = (m.get("mask") or {}).get("size", 0)
@@ -98,21 +116,23 @@ def latent_attention(hs, W, pre, m, eps):
     uk, uv = W[pre + "uk"].reshape(H, D, R), W[pre + "uv"].reshape(H, Dv, R)
     out = []
     for i, h in enumerate(hs):
-        heads = np.zeros((H, Dv))
-        for a in range(H):
-            qn = qs[i][a, :D]
-            qr = rotate(qs[i][a, D:], i, freqs, amp, rot["dims"], False)
-            js = list(visible(i, window))
-            sc = np.array([(qn @ (uk[a] @ lat[j]) + qr @ krot[j]) * m["scale"] for j in js])
-            sink = float(W[pre + "sink"][a])
-            top = max(sc.max(), sink)
-            e = np.exp(sc - top)
-            den = e.sum() + math.exp(sink - top)
-            for wgt, j in zip(e / den, js):
-                heads[a] += wgt * (uv[a] @ lat[j])
+        qr = np.stack([rotate(qs[i][a, D:], i, freqs, amp, rot["dims"], False) for a in range(H)])
+        heads = latent_core(qs[i][:, :D], qr, lat, krot, uk, uv, i, window, m["scale"],
+                            W[pre + "sink"])
         gated = heads.reshape(-1) * sigmoid(W[pre + "g"] @ h)
         out.append(W[pre + "o"] @ gated)
     return out
+
+
+def sigmoid_core(q, ks, vs, i, H, G, window, scale, pb):
+    """Heads [H, Dv] of position i: every visible key j weighs sigmoid(q_h . k_j scale + pb_h).
+    q [H, D]; ks[j] [G, D]; vs[j] [G, Dv]."""
+    heads = np.zeros((H, vs[0].shape[1]))
+    for a in range(H):
+        b = a // (H // G)
+        for j in visible(i, window):
+            heads[a] += sigmoid(float(q[a] @ ks[j][b]) * scale + float(pb[a])) * vs[j][b]
+    return heads
 
 
 def sigmoid_attention(hs, W, pre, m, eps):
@@ -131,12 +151,7 @@ def sigmoid_attention(hs, W, pre, m, eps):
         vs.append((W[pre + "v"] @ h).reshape(G, Dv))
     out = []
     for i in range(len(hs)):
-        heads = np.zeros((H, Dv))
-        for a in range(H):
-            b = a // (H // G)
-            for j in visible(i, window):
-                s = float(qs[i][a] @ ks[j][b]) * m["scale"] + float(W[pre + "pb"][a])
-                heads[a] += sigmoid(s) * vs[j][b]
+        heads = sigmoid_core(qs[i], ks, vs, i, H, G, window, m["scale"], W[pre + "pb"])
         out.append(W[pre + "o"] @ heads.reshape(-1))
     return out
 
