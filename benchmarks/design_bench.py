@@ -10,6 +10,9 @@ For each size the two engines are built one after the other on the same device:
 attention, grouped norms, a looped stack, gated GELU feed-forward) beside a Mistral-style decoder
 (sliding-window grouped-query attention + SwiGLU) with the same width, number of layer runs, head
 count, head size, window and ff.
+``--design gapidra`` runs the Gapidra design (parallel sublayers on one norm; sigmoid window
+attention and windowed latent attention with sinks, alternating; ungated xIELU feed-forward)
+beside the same Mistral-style decoder at equal width, depth, heads, head size, window and ff.
 Prefill: ``--design-prompts`` prompts of ``--design-prompt-len`` tokens, one sampled token each.
 Decode: ``--design-users`` sequences of 128 prompt tokens generating ``--design-gen`` tokens; the
 decode rate is the extra tokens over the extra time against the same run with one token.
@@ -103,6 +106,33 @@ def mistral_config(z: dict) -> dict:
             "max_position_embeddings": 32768, "rms_norm_eps": 1e-5, "rope_theta": 1e6}
 
 
+GSIZES = {
+    # name: width, heads, kv heads, head dim, latent rank, rotary part, window, ff, vocab
+    "gs": dict(width=1024, heads=8, kv_heads=2, dim=128, kv_rank=256, rot=64, window=1024, ff=4096,
+               vocab=32000),
+    "gm": dict(width=2048, heads=16, kv_heads=4, dim=128, kv_rank=512, rot=64, window=1024,
+               ff=8192, vocab=32000),
+}
+
+
+def gapidra_config(z: dict) -> dict:
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    mlp = {"kind": "dense", "ff": z["ff"]}
+    att = {"type": "attention", "mlp": mlp,
+           "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
+                     "mask": {"size": z["window"]},
+                     "rot": {"base": 1e6, "dims": D // 2,
+                             "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0,
+                                         "slow": 1.0}}}}
+    lat = {"type": "latent_attention", "mlp": mlp,
+           "mixer": {"heads": H, "dim": D - z["rot"], "rot_dim": z["rot"], "vdim": D,
+                     "kv_rank": z["kv_rank"], "scale": D ** -0.5, "mask": {"size": z["window"]},
+                     "rot": {"base": 1e6, "dims": z["rot"]}}}
+    return {"architecture": "Gapidra", "vocab": z["vocab"], "width": z["width"],
+            "norm": {"eps": 1e-5}, "embedding": {"scale": z["width"] ** 0.5},
+            "layers": [att, lat, lat, att, lat, att]}
+
+
 def _measure(cfg_dict: dict, a) -> dict:
     import torch
 
@@ -152,12 +182,17 @@ def _measure(cfg_dict: dict, a) -> dict:
 
 def run(a) -> int:
     rows = []
-    vedadra = getattr(a, "design", "sekolorn") == "vedadra"
-    for name in (a.design_sizes or ("vs,vm" if vedadra else "s,s6")).split(","):
+    design = getattr(a, "design", "sekolorn")
+    vedadra = design == "vedadra"
+    default = {"vedadra": "vs,vm", "gapidra": "gs,gm"}.get(design, "s,s6")
+    for name in (a.design_sizes or default).split(","):
         if name in GATED:
             raise SystemExit(f"design size {name!r} is switched off (see GATED in "
                              "benchmarks/design_bench.py); run s or s6")
-        if vedadra:
+        if design == "gapidra":
+            z = dict(GSIZES[name], layers=6)
+            pair = (("Gapidra", gapidra_config(z)), ("Mistral-style", mistral_config(z)))
+        elif vedadra:
             z = dict(VSIZES[name], layers=6)
             pair = (("Vedadra", vedadra_config(z)), ("Mistral-style", mistral_config(z)))
         else:
@@ -202,6 +237,8 @@ def kernel_rates(a) -> int:
 
     if getattr(a, "design", "sekolorn") == "vedadra":
         return window_kernel_rates(a)
+    if getattr(a, "design", "sekolorn") == "gapidra":
+        return gapidra_kernel_rates(a)
     from enterprise_inference_amd.ops import attention as A
     from enterprise_inference_amd.ops import latent_attention as LA
     from enterprise_inference_amd.ops import wkv as WK
@@ -395,5 +432,126 @@ def window_kernel_rates(a) -> int:
     for r_ in rows:
         print(json.dumps(r_), flush=True)
     print(json.dumps({"metric": "design_kernel_rates", "design": "vedadra", "rows": rows}),
+          flush=True)
+    return 0
+
+
+def gapidra_kernel_rates(a) -> int:
+    """Achieved rates of the Gapidra kernels beside the sliding-window paged kernels of the Llama
+    path at equal heads, head size, window and lengths: sigmoid window attention and windowed
+    latent attention with sinks -- prefill in useful TFLOP/s (2 (Dqk + Dv) per visible query-key
+    pair and head; the second product's remainder pass is not counted), decode in cache bytes of
+    the visible keys per second -- and the layer boundary (two sublayer outputs + residual + next
+    norm on an fp32 stream) beside the bf16 fused add + RMS norm in bytes moved per second.  One
+    JSON line per kernel."""
+    import torch
+
+    from enterprise_inference_amd.ops import attention as A
+    from enterprise_inference_amd.ops import latent_attention as LA
+    from enterprise_inference_amd.ops import norm as N
+    from enterprise_inference_amd.ops import window_attention as WA
+    from enterprise_inference_amd.ops.rotary import rotary_frequencies
+
+    dev, bf = "cuda", torch.bfloat16
+    bs, win, T = 128, 1024, 4096
+    rows = []
+    pairs = T * win - win * (win - 1) // 2                     # visible (query, key) pairs
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    B, L = 64, 4096
+    nb, nbd = T // bs, B * L // bs
+    pos = torch.arange(T, dtype=torch.int32, device=dev)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+    md = A.AttentionMetadata(
+        num_decode=0, num_prefill_tokens=T, slot_mapping=pos, positions=pos,
+        prefill_block_tables=bt, prefill_seq_lens=i32([T]), prefill_cu_q=i32([0, T]),
+        prefill_q_lens=[T])
+    btd = torch.arange(nbd, dtype=torch.int32, device=dev).view(B, L // bs)
+    posd = torch.full((B,), L - 1, dtype=torch.int32, device=dev)
+    mdd = A.AttentionMetadata(num_decode=B, num_prefill_tokens=0, slot_mapping=posd,
+                              positions=posd, decode_block_tables=btd,
+                              decode_seq_lens=i32([L] * B))
+    for H, G, R, rd in ((8, 2, 256, 64), (16, 4, 512, 64)):
+        D = Dv = 128
+        # sigmoid window attention
+        spec = WA.WindowSpec(H, G, 1, D, Dv, win, 0, mult=torch.full((H,), D ** -0.5, device=dev),
+                             weights=1, bias=torch.full((H,), -4.0, device=dev))
+        kc = torch.randn(nb, bs, G * D, device=dev).to(bf)
+        vc = torch.randn(nb, G * Dv, bs, device=dev).to(bf)
+        q = torch.randn(T, H * D, device=dev).to(bf)
+        t = _time(lambda: WA.window_attention(q, kc, vc, md, spec, None))
+        rows.append({"kernel": "window_attn prefill (sigmoid)", "heads": H, "kv_heads": G,
+                     "dim": D, "vdim": Dv, "window": win, "tokens": T, "ms": t * 1e3,
+                     "mfma": WA.mfma_ok(spec, bf, bs),
+                     "tflops": 2.0 * (D + Dv) * H * pairs / t / 1e12})
+        kcd = torch.randn(nbd, bs, G * D, device=dev).to(bf)
+        vcd = torch.randn(nbd, G * Dv, bs, device=dev).to(bf)
+        qd = q[:B].contiguous()
+        t = _time(lambda: WA.window_attention(qd, kcd, vcd, mdd, spec, None))
+        rows.append({"kernel": "window_attn decode (sigmoid)", "heads": H, "kv_heads": G,
+                     "batch": B, "context": L, "window": win, "ms": t * 1e3,
+                     "cache_GBps": B * win * G * (D + Dv) * 2 / t / 1e9})
+        del kcd, vcd
+        # windowed latent attention with sinks (absorbed form: Dqk = R + rd, Dv = R)
+        inv, amp = rotary_frequencies(rd, 1e6, None, dev)
+        sink = torch.zeros(H, device=dev)
+        cache = torch.randn(nb, bs, R + rd, device=dev).to(bf)
+        qa = torch.randn(T, H, R, device=dev).to(bf) * 0.1
+        qr = torch.randn(T, H, rd, device=dev).to(bf) * 0.1
+        qb = LA.query_block(H, R, rd, bf)
+        work = LA.build_work([T], qb)
+        mdl = A.AttentionMetadata(
+            num_decode=0, num_prefill_tokens=T, slot_mapping=pos, positions=pos,
+            prefill_block_tables=bt, prefill_seq_lens=i32([T]), prefill_cu_q=i32([0, T]),
+            prefill_work=i32(work), prefill_n_work=len(work) // 2, prefill_qblock=qb)
+        t = _time(lambda: LA.latent_attention(qa, qr, inv, rd, cache, mdl, None, 0.1, win, sink,
+                                              True, amp))
+        rows.append({"kernel": "latent_attn prefill (window, sink)", "heads": H, "kv_rank": R,
+                     "rot": rd, "window": win, "tokens": T, "ms": t * 1e3,
+                     "tflops": 2.0 * (2 * R + rd) * H * pairs / t / 1e12})
+        cache_d = torch.randn(nbd, bs, R + rd, device=dev).to(bf)
+        qad, qrd = qa[:B].contiguous(), qr[:B].contiguous()
+        t = _time(lambda: LA.latent_attention(qad, qrd, inv, rd, cache_d, mdd, None, 0.1, win, sink,
+                                              True, amp))
+        rows.append({"kernel": "latent_attn decode (window, sink)", "heads": H, "kv_rank": R,
+                     "batch": B, "context": L, "window": win, "ms": t * 1e3,
+                     "cache_GBps": B * win * (R + rd) * 2 / t / 1e9})
+        del cache_d
+        # the like kernels: sliding-window paged prefill (flash form) and decode, D = 128
+        kc = torch.randn(nb, G, bs, D, device=dev).to(bf)
+        vc = torch.randn(nb, G, D, bs, device=dev).to(bf)
+        q3 = torch.randn(T, H, D, device=dev).to(bf) * 0.1
+        qb2 = A.prefill_query_block(H, G, D, block_size=bs)
+        w2 = A.build_prefill_work([T], qb2)
+        wt = i32(w2)
+        t = _time(lambda: A.paged_prefill(q3, kc, vc, bt, i32([T]), i32([0, T]), wt, len(w2) // 2,
+                                          0.1, sliding_window=win))
+        rows.append({"kernel": "paged_prefill (flash, sliding window)", "heads": H, "kv_heads": G,
+                     "head_dim": D, "window": win, "tokens": T, "ms": t * 1e3,
+                     "tflops": 2.0 * 2 * D * H * pairs / t / 1e12})
+        kcd = torch.randn(nbd, G, bs, D, device=dev).to(bf)
+        vcd = torch.randn(nbd, G, D, bs, device=dev).to(bf)
+        lens = i32([L] * B)
+        qd3 = q3[:B].contiguous()
+        t = _time(lambda: A.paged_decode(qd3, kcd, vcd, btd, lens, 0.1, sliding_window=win))
+        rows.append({"kernel": "paged_decode (sliding window)", "heads": H, "kv_heads": G,
+                     "batch": B, "context": L, "window": win, "ms": t * 1e3,
+                     "cache_GBps": B * win * G * D * 2 * 2 / t / 1e9})
+        del kcd, vcd
+    for W in (2048, 4096):
+        Tn = 8192
+        x = torch.randn(Tn, W, device=dev)
+        y1 = torch.randn(Tn, W, device=dev).to(bf)
+        y2 = torch.randn(Tn, W, device=dev).to(bf)
+        w1 = torch.ones(W, device=dev).to(bf)
+        t = _time(lambda: N.residual_rms_step(x, 1e-5, (y1, y2), w1))
+        rows.append({"kernel": "residual_rms_step (2 outputs)", "width": W, "rows": Tn,
+                     "ms": t * 1e3, "GBps": Tn * W * (2 + 2 + 4 + 4 + 2) / t / 1e9})
+        res = torch.randn(Tn, W, device=dev).to(bf)
+        t = _time(lambda: N.fused_add_rms_norm(y1, res, w1, 1e-5))
+        rows.append({"kernel": "fused_add_rms_norm", "width": W, "rows": Tn, "ms": t * 1e3,
+                     "GBps": Tn * W * (2 + 2 + 2 + 2) / t / 1e9})
+    for r_ in rows:
+        print(json.dumps(r_), flush=True)
+    print(json.dumps({"metric": "design_kernel_rates", "design": "gapidra", "rows": rows}),
           flush=True)
     return 0

@@ -73,8 +73,7 @@ def xielu(x, pq: torch.Tensor) -> torch.Tensor:
     from .gemm import SplitK
     split = isinstance(x, SplitK)
     if split and not (x.part.is_cuda and x.bias is None and x.N % 4 == 0 and x.part.is_contiguous()):
-        x = x.materialize() if x.part.is_cuda else (x.part.sum(0) + (
-            x.bias.float() if x.bias is not None else 0.0)).to(pq.dtype)
+        x = (x.part.sum(0) + (x.bias.float() if x.bias is not None else 0.0)).to(pq.dtype)
         split = False
     if not split and not use_hip(x):
         z = x.float()

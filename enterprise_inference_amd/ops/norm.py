@@ -193,8 +193,12 @@ def residual_rms_step(x: torch.Tensor, eps: float, ys=(), w_next: Optional[torch
         return y.float()
 
     if use_hip(x) and W % 4:
-        # the kernel sums partials in 16-byte units; no GEMM of the framework produces other widths
-        ys = [dense(y) if isinstance(y, SplitK) else y for y in ys]
+        # the kernel sums partials in 16-byte units; other widths (no GEMM of the framework
+        # produces them) join the stream through the unfused fp32 sum
+        for y in ys:
+            if isinstance(y, SplitK):
+                x += dense(y)
+        ys = [y for y in ys if not isinstance(y, SplitK)]
     if not use_hip(x):
         for y in ys:
             x += dense(y)
