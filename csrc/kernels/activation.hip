@@ -156,10 +156,23 @@ EIA_DEV float xielu_f(float z, float ap, float aq) {
   return z > 0.f ? ap * z * z + 0.5f * z : aq * (expm1f(z) - z) + 0.5f * z;
 }
 
+// four consecutive elements of a bf16 or fp32 row (8- / 16-byte accesses)
+template <typename T> EIA_DEV f32x4 act_ld4(const T* p);
+template <> EIA_DEV f32x4 act_ld4<bf16_t>(const bf16_t* p) {
+  const bf16x4 v = *reinterpret_cast<const bf16x4*>(p);
+  return f32x4{(float)v[0], (float)v[1], (float)v[2], (float)v[3]};
+}
+template <> EIA_DEV f32x4 act_ld4<float>(const float* p) { return *reinterpret_cast<const f32x4*>(p); }
+template <typename T> EIA_DEV void act_st4(T* p, f32x4 v);
+template <> EIA_DEV void act_st4<bf16_t>(bf16_t* p, f32x4 v) {
+  *reinterpret_cast<bf16x4*>(p) = bf16x4{f2bf(v[0]), f2bf(v[1]), f2bf(v[2]), f2bf(v[3])};
+}
+template <> EIA_DEV void act_st4<float>(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+
 template <typename T>
 __global__ void __launch_bounds__(256)
 xielu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ part, int sk,
-             const T* __restrict__ pq, T* __restrict__ out, long ldo, int rows, int F) {
+             const T* __restrict__ pq, T* __restrict__ out, long ldo, int rows, int F, int vec) {
   const float ap = softplus_f(ld_f32<T>(pq, 0)), aq = 0.5f + softplus_f(ld_f32<T>(pq, 1));
   if (part) {
     const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
@@ -169,8 +182,22 @@ xielu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ part, 
     const float* p = part + idx;
     f32x4 v = *reinterpret_cast<const f32x4*>(p);
     for (int z = 1; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * slab);
+    if (vec) {
+      act_st4<T>(out + (long)row * ldo + col, f32x4{xielu_f(v[0], ap, aq), xielu_f(v[1], ap, aq),
+                                                    xielu_f(v[2], ap, aq), xielu_f(v[3], ap, aq)});
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < 4; ++i) st_f32<T>(out + (long)row * ldo, col + i, xielu_f(v[i], ap, aq));
+    return;
+  }
+  if (vec) {                                         // F, ldx, ldo multiples of 4
+    const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (idx >= (long)rows * F) return;
+    const int row = idx / F, col = idx % F;
+    const f32x4 v = act_ld4<T>(x + (long)row * ldx + col);
+    act_st4<T>(out + (long)row * ldo + col, f32x4{xielu_f(v[0], ap, aq), xielu_f(v[1], ap, aq),
+                                                  xielu_f(v[2], ap, aq), xielu_f(v[3], ap, aq)});
     return;
   }
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
@@ -185,40 +212,66 @@ EIA_API int eia_xielu(const void* x, long ldx, const float* part, int sk, const 
       (part && (sk < 1 || F % 4)))
     return EIA_BAD_SHAPE;
   if (rows == 0) return EIA_OK;
-  const long n = part ? (long)rows * F / 4 : (long)rows * F;
+  const int esz = is_bf16 ? 2 : 4;
+  const int vec = F % 4 == 0 && ldx % 4 == 0 && ldo % 4 == 0 &&
+                  ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(out)) % (4 * esz)) == 0;
+  const long n = (part || vec) ? (long)rows * F / 4 : (long)rows * F;
   dim3 grid((unsigned)((n + 255) / 256)), block(256);
   if (is_bf16)
     hipLaunchKernelGGL(xielu_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)x, ldx, part, sk,
-                       (const bf16_t*)pq, (bf16_t*)out, ldo, rows, F);
+                       (const bf16_t*)pq, (bf16_t*)out, ldo, rows, F, vec);
   else
     hipLaunchKernelGGL(xielu_kernel<float>, grid, block, 0, st, (const float*)x, ldx, part, sk,
-                       (const float*)pq, (float*)out, ldo, rows, F);
+                       (const float*)pq, (float*)out, ldo, rows, F, vec);
   EIA_LAUNCH_CHECK();
 }
 
-// out[t, c] = a[t, c] * sigmoid(g[t, c]); a and g are rows with their own strides (either may be
-// a column slice of a wider row), fp32 inside.
+// out[t, c] = a(t, c) * sigmoid(g[t, c]), fp32 inside.  g and out are rows with their own strides
+// (g may be a column slice of a wider row); a is either such a row too (V == N) or laid out head
+// by head, a(t, h * V + v) = a[h * a_sh + t * lda + v] (the output of a batched product over
+// heads), so the heads are concatenated here without a transposing copy.  vec: four columns per
+// thread (V, the strides and the pointers allow 8- / 16-byte accesses).
 template <typename T>
 __global__ void __launch_bounds__(256)
-sigmoid_gate_kernel(const T* __restrict__ a, long lda, const T* __restrict__ g, long ldg,
-                    T* __restrict__ out, long ldo, int rows, int N) {
+sigmoid_gate_kernel(const T* __restrict__ a, long lda, long a_sh, int V, const T* __restrict__ g,
+                    long ldg, T* __restrict__ out, long ldo, int rows, int N, int vec) {
+  if (vec) {
+    const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (idx >= (long)rows * N) return;
+    const int row = idx / N, col = idx % N;
+    const int h = col / V;
+    const f32x4 av = act_ld4<T>(a + h * a_sh + (long)row * lda + (col - h * V));
+    const f32x4 gv = act_ld4<T>(g + (long)row * ldg + col);
+    f32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = av[i] / (1.0f + expf(-gv[i]));
+    act_st4<T>(out + (long)row * ldo + col, o);
+    return;
+  }
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   if (idx >= (long)rows * N) return;
   const int row = idx / N, col = idx % N;
+  const int h = col / V;
   const float gv = ld_f32<T>(g + (long)row * ldg, col);
-  st_f32<T>(out + (long)row * ldo, col, ld_f32<T>(a + (long)row * lda, col) / (1.0f + expf(-gv)));
+  st_f32<T>(out + (long)row * ldo, col,
+            ld_f32<T>(a + h * a_sh + (long)row * lda, col - h * V) / (1.0f + expf(-gv)));
 }
 
-EIA_API int eia_sigmoid_gate(const void* a, long lda, const void* g, long ldg, void* out, long ldo,
-                             int rows, int N, int is_bf16, hipStream_t st) {
-  if (rows < 0 || N < 1 || !a || !g || !out) return EIA_BAD_SHAPE;
+EIA_API int eia_sigmoid_gate(const void* a, long lda, long a_sh, int V, const void* g, long ldg,
+                             void* out, long ldo, int rows, int N, int is_bf16, hipStream_t st) {
+  if (rows < 0 || N < 1 || V < 1 || N % V || !a || !g || !out) return EIA_BAD_SHAPE;
   if (rows == 0) return EIA_OK;
-  dim3 grid((unsigned)(((long)rows * N + 255) / 256)), block(256);
+  const int esz = is_bf16 ? 2 : 4;
+  const int vec = V % 4 == 0 && lda % 4 == 0 && a_sh % 4 == 0 && ldg % 4 == 0 && ldo % 4 == 0 &&
+                  ((reinterpret_cast<uintptr_t>(a) | reinterpret_cast<uintptr_t>(g) |
+                    reinterpret_cast<uintptr_t>(out)) % (4 * esz)) == 0;
+  const long n = vec ? (long)rows * N / 4 : (long)rows * N;
+  dim3 grid((unsigned)((n + 255) / 256)), block(256);
   if (is_bf16)
-    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)a, lda,
-                       (const bf16_t*)g, ldg, (bf16_t*)out, ldo, rows, N);
+    hipLaunchKernelGGL(sigmoid_gate_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)a, lda, a_sh,
+                       V, (const bf16_t*)g, ldg, (bf16_t*)out, ldo, rows, N, vec);
   else
-    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, block, 0, st, (const float*)a, lda,
-                       (const float*)g, ldg, (float*)out, ldo, rows, N);
+    hipLaunchKernelGGL(sigmoid_gate_kernel<float>, grid, block, 0, st, (const float*)a, lda, a_sh,
+                       V, (const float*)g, ldg, (float*)out, ldo, rows, N, vec);
   EIA_LAUNCH_CHECK();
 }

@@ -32,6 +32,21 @@ EIA_DEV float lat_rotated(const T* src, int d, int rot_dims, bool half, float am
   return second ? (w * cs + u * sn) : (u * cs - w * sn);
 }
 
+// Entries dd0 .. dd0 + 7 of a rotary query part after the rotation (entries past rot_dims pass
+// unchanged).  Not inlined: one copy of the sine / cosine code per kernel.
+__device__ __attribute__((noinline)) bf16x8
+lat_rot_chunk(const bf16_t* qr, int dd0, int rot_dims, bool half, float amp, float pos,
+              const float* __restrict__ inv_freq) {
+  bf16x8 v;
+#pragma unroll 1
+  for (int e = 0; e < 8; ++e) {
+    const int dd = dd0 + e;
+    v[e] = f2bf(dd < rot_dims ? lat_rotated<bf16_t>(qr, dd, rot_dims, half, amp, pos, inv_freq)
+                              : bf2f(qr[dd]));
+  }
+  return v;
+}
+
 // ------------------------------------------------------------------------------------------ prep
 // fused [T, ld]: columns [q_off, q_off+q_rank) query latent, [c_off, c_off+R) KV latent,
 // [kr_off, kr_off+rd) shared rotary key part.  q_rank == 0: no query latent; cache == nullptr:
@@ -100,6 +115,11 @@ EIA_API int eia_latent_prep(const void* fused, long ld, int q_off, int q_rank, c
 }
 
 // ------------------------------------------------------------------------------------- attention
+// Key partitions a decode row uses out of the launch's grid.z: at least two 32-key units each.
+EIA_DEV int lat_parts(int nparts, int kmin, int kmax) {
+  return min(nparts, max(1, ((kmax - kmin + 31) >> 5) >> 1));
+}
+
 #define LAT_ACC_MAX 32     // fp32 accumulators per thread: QB * HB * R <= 256 * LAT_ACC_MAX
 
 struct LatentAttnArgs {
@@ -387,25 +407,27 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
   {
     const bf16_t* qa = static_cast<const bf16_t*>(a.qa) + row * a.qa_st + (long)h * a.qa_sh;
     const bf16_t* qr = static_cast<const bf16_t*>(a.qr) + row * a.qr_st + (long)h * a.qr_sh;
+    // R % 8 == 0: a lane's 8-entry chunk lies wholly in the absorbed part (one 16-byte load when
+    // the rows are aligned) or wholly in the rotary part (rotated by a called, rolled helper:
+    // the sine / cosine code exists once, not once per entry of the unrolled operand)
+    const bool qvec = ((reinterpret_cast<uintptr_t>(a.qa) | (uintptr_t)(a.qa_st * 2) |
+                        (uintptr_t)(a.qa_sh * 2)) & 15) == 0;
 #pragma unroll
     for (int s = 0; s < NKMAX; ++s) {
+      const int d0 = s * 32 + 8 * g;
+      bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (row_ok && s < nk && d0 < Dk) {
+        if (d0 >= a.R) {
+          v = lat_rot_chunk(qr, d0 - a.R, a.rot_dims, a.rot_half != 0, a.rot_amp, (float)qpos,
+                            a.inv_freq);
+        } else if (qvec) {
+          v = *reinterpret_cast<const bf16x8*>(qa + d0);
+        } else {
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const int d = s * 32 + 8 * g + e;
-        float v = 0.f;
-        if (row_ok && s < nk && d < Dk) {
-          if (d < a.R) {
-            v = bf2f(qa[d]);
-          } else {
-            const int dd = d - a.R;
-            v = dd < a.rot_dims
-                ? lat_rotated<bf16_t>(qr, dd, a.rot_dims, a.rot_half != 0, a.rot_amp, (float)qpos,
-                                      a.inv_freq)
-                : bf2f(qr[dd]);
-          }
+          for (int e = 0; e < 8; ++e) v[e] = qa[d0 + e];
         }
-        qf[s][e] = f2bf(v);
       }
+      qf[s] = v;
     }
   }
   constexpr int NACC = SPLITV ? (NCMAX + NW - 1) / NW : NCMAX;   // column tiles of this wave
@@ -419,12 +441,16 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
   // first 32-key unit that holds a key some row of the tile sees
   const int kmin = a.window > 0 ? (max(0, a.positions[row0] - a.window + 1) & ~31) : 0;
   int k_begin = kmin, k_end = kmax;
-  if (a.nparts > 1) {                                      // this partition's run of 32-key units
+  // partitions this row really uses: at least two 32-key units each (decided here and, the same
+  // way, in the merge kernel), so short contexts do not pay for idle partitions
+  const int np = lat_parts(a.nparts, kmin, kmax);
+  if (np > 1) {                                            // this partition's run of 32-key units
     const int units = (kmax - kmin + 31) >> 5;
-    const int per = (units + a.nparts - 1) / a.nparts;
+    const int per = (units + np - 1) / np;
     k_begin = kmin + (min((int)blockIdx.z * per, units) << 5);
     k_end = min(kmax, kmin + (((int)blockIdx.z + 1) * per << 5));
   }
+  if ((int)blockIdx.z >= np) return;                       // (whole workgroup)
   const int wlo = a.window > 0 ? qpos - a.window + 1 : 0;   // first key this lane's row sees
   const int cpr = Dkp >> 3;                                // 16-byte chunks per (padded) key row
   const int nchunk = 32 * cpr;
@@ -533,7 +559,7 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
     __syncthreads();
   }
   if (!row_ok) return;
-  if (a.nparts > 1) {
+  if (np > 1) {
     const long pr = ((long)row * a.H + h) * a.nparts + blockIdx.z;
     float* pa = a.part_acc + pr * a.R;
 #pragma unroll
@@ -574,32 +600,40 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
 }
 
 // Merge of the decode partitions: out = sum_p acc_p 2^(m_p - M) / sum_p l_p 2^(m_p - M), times
-// the head gate.  One workgroup per (row, head), threads over the latent columns.
+// the head gate.  One workgroup per (row, head); lane p first turns partition p's (max, sum) into
+// its weight, then the threads sum the latent columns over the partitions with independent loads
+// (nparts <= 64).  Rows whose context is too short for two partitions were finished by the
+// attention kernel itself.
 __global__ void __launch_bounds__(128)
 latent_merge_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                    int nparts, const int* __restrict__ seq_lens, const bf16_t* __restrict__ gate,
-                    long gate_st, const float* __restrict__ sink, bf16_t* __restrict__ out,
-                    long out_st, long out_sh, int H, int R) {
-  const int row = blockIdx.x, h = blockIdx.y;
+                    int nparts, const int* __restrict__ seq_lens, const int* __restrict__ positions,
+                    int window, const bf16_t* __restrict__ gate, long gate_st,
+                    const float* __restrict__ sink, bf16_t* __restrict__ out, long out_st,
+                    long out_sh, int H, int R) {
+  const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63;
   if (seq_lens && seq_lens[row] <= 0) return;
+  const int kmax = positions[row] + 1;
+  const int kmin = window > 0 ? (max(0, kmax - window) & ~31) : 0;
+  const int np = lat_parts(nparts, kmin, kmax);
+  if (np == 1) return;
   const long pr = ((long)row * H + h) * nparts;
-  float M = -INFINITY;
-  for (int p = 0; p < nparts; ++p) M = fmaxf(M, part_ml[2 * (pr + p)]);
-  float L = 0.f;
-  for (int p = 0; p < nparts; ++p) {
-    const float m = part_ml[2 * (pr + p)];
-    if (m != -INFINITY) L += part_ml[2 * (pr + p) + 1] * exp2f(m - M);
-  }
+  const float mp = lane < np ? part_ml[2 * (pr + lane)] : -INFINITY;
+  const float lp = lane < np ? part_ml[2 * (pr + lane) + 1] : 0.f;
+  const float M = wave_max(mp);
+  const float wp = (mp == -INFINITY) ? 0.f : exp2f(mp - M);
+  float L = wave_sum(lp * wp);
   if (sink && M != -INFINITY) L += exp2f(sink[h] * 1.4426950408889634f - M);
   float f = L > 0.f ? 1.0f / L : 0.f;
   if (gate) f *= 1.0f / (1.0f + expf(-bf2f(gate[row * gate_st + h])));
-  for (int c = threadIdx.x; c < R; c += blockDim.x) {
+  for (int c0 = 0; c0 < R; c0 += blockDim.x) {
+    const int c = c0 + threadIdx.x;
     float v = 0.f;
-    for (int p = 0; p < nparts; ++p) {
-      const float m = part_ml[2 * (pr + p)];
-      if (m != -INFINITY) v += part_acc[(pr + p) * R + c] * exp2f(m - M);
+#pragma unroll 4
+    for (int p = 0; p < np; ++p) {
+      const float w = __shfl(wp, p, 64);
+      if (c < R) v += part_acc[(pr + p) * R + c] * w;
     }
-    out[row * out_st + h * out_sh + c] = f2bf(v * f);
+    if (c < R) out[row * out_st + h * out_sh + c] = f2bf(v * f);
   }
 }
 
@@ -659,7 +693,7 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
 #undef LAT_MFMA
   if (nparts > 1)
     hipLaunchKernelGGL(latent_merge_kernel, dim3(n_items, H), dim3(128), 0, st, part_acc, part_ml,
-                       nparts, seq_lens, static_cast<const bf16_t*>(gate), gate_st, sink,
-                       static_cast<bf16_t*>(out), out_st, out_sh, H, R);
+                       nparts, seq_lens, positions, window, static_cast<const bf16_t*>(gate),
+                       gate_st, sink, static_cast<bf16_t*>(out), out_st, out_sh, H, R);
   EIA_LAUNCH_CHECK();
 }

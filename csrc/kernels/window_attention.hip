@@ -136,6 +136,15 @@ qk_rope_cache_kernel(const T* __restrict__ fused, long ld, const float* __restri
   const long t = blockIdx.x;
   const long slot = slots ? (long)slots[t] : -1;
   extern __shared__ float rsum[];                   // [ld] when the row arrives as partials
+  const int hd = rot_dims >> 1;
+  // the token's cos / sin (times amp), once per pair index, behind the summed row
+  float* cs_t = rsum + (part ? ld : 0);             // [hd] cos, then [hd] sin
+  for (int i = threadIdx.x; i < hd; i += blockDim.x) {
+    float sn, cs;
+    sincosf((float)positions[t] * inv_freq[i], &sn, &cs);
+    cs_t[i] = cs * amp;
+    cs_t[hd + i] = sn * amp;
+  }
   if (part) {
     for (int c = 4 * threadIdx.x; c < (int)ld; c += 4 * blockDim.x) {
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
@@ -146,11 +155,9 @@ qk_rope_cache_kernel(const T* __restrict__ fused, long ld, const float* __restri
       for (int z = 0; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * pstride);
       *reinterpret_cast<f32x4*>(rsum + c) = v;
     }
-    __syncthreads();
   }
+  __syncthreads();
   auto val = [&](int c) -> float { return fused ? ld_f32<T>(fused + t * ld, c) : rsum[c]; };
-  const float pos = (float)positions[t];
-  const int hd = rot_dims >> 1;
   for (int side = 0; side < 2; ++side) {
     if (side == 1 && slot < 0) break;               // (uniform per workgroup)
     const int n = (side ? MK : MQ) * D, off = side ? k_off : q_off;
@@ -174,10 +181,7 @@ qk_rope_cache_kernel(const T* __restrict__ fused, long ld, const float* __restri
       if (d < rot_dims) {
         const int i = half ? (d < hd ? d : d - hd) : (d >> 1);
         const bool second = half ? d >= hd : (d & 1);
-        float sn, cs;
-        sincosf(pos * inv_freq[i], &sn, &cs);
-        sn *= amp;
-        cs *= amp;
+        const float cs = cs_t[i], sn = cs_t[hd + i];
         const int da = half ? i : 2 * i, db = half ? i + hd : 2 * i + 1;
         const float o = normed(c0 + (second ? da : db));    // the pair's other entry
         v = second ? (v * cs + o * sn) : (v * cs - o * sn);
@@ -203,7 +207,7 @@ EIA_API int eia_qk_rope_cache(const void* fused, long ld, const float* part, int
     return EIA_BAD_SHAPE;
   if (T == 0) return EIA_OK;
   const long ps = (long)T * ld;
-  const size_t lds = part ? sizeof(float) * ld : 0;
+  const size_t lds = (part ? sizeof(float) * ld : 0) + sizeof(float) * rot_dims;
   if (lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (is_bf16)
     hipLaunchKernelGGL((qk_rope_cache_kernel<bf16_t>), dim3(T), dim3(256), lds, st,

@@ -89,7 +89,7 @@ _SIGNATURES = {
                           I, F, I, I, S],
     "eia_add_rms": [P, L, P, I, P, P, L, P, I, P, P, P, P, L, F, I, I, I, S],
     "eia_xielu": [P, L, P, I, P, P, L, I, I, I, S],
-    "eia_sigmoid_gate": [P, L, P, L, P, L, I, I, I, S],
+    "eia_sigmoid_gate": [P, L, L, I, P, L, P, L, I, I, I, S],
     "eia_window_attn_mfma_ok": [I, I, I, I, I, I, I],
     "eia_ar_alloc": [P, L],
     "eia_moe_splitk_norm_route": [P, I, I, I, P, P, F, P, L, P, I, I, I, I, P, P, P, S],

@@ -155,9 +155,10 @@ class LatentAttentionMixer(nn.Module):
                                        self.rot_amp)
         # value up-projection of the attended latent, heads concatenated
         o = torch.bmm(lat.transpose(0, 1), self.uv.view(H, self.vdim, R).transpose(1, 2))
-        o = o.transpose(0, 1).reshape(T, H * self.vdim)
-        if self.gate == "element":
+        if self.gate == "element":      # [H, T, vdim] -> gated [T, H * vdim] in one pass
             o = act_ops.sigmoid_gate(o, fused[:, g0:g0 + self.gate_rows])
+        else:
+            o = o.transpose(0, 1).reshape(T, H * self.vdim)
         return gemm.linear(o, self.o, defer_reduce=self.defer_out)
 
 

@@ -100,16 +100,27 @@ def xielu(x, pq: torch.Tensor) -> torch.Tensor:
 
 
 def sigmoid_gate(a: torch.Tensor, gate: torch.Tensor) -> torch.Tensor:
-    """a * sigmoid(gate), element by element (fp32 inside); a, gate [T, N] rows with a contiguous
-    last dim (either may be a column slice of a wider row) -> [T, N] contiguous."""
-    if not use_hip(a, gate):
-        return (a.float() * torch.sigmoid(gate.float())).to(a.dtype)
-    require(a.dim() == 2 and a.shape == gate.shape and a.stride(1) == 1 and gate.stride(1) == 1
-            and a.dtype == gate.dtype and a.dtype in (torch.bfloat16, torch.float32),
-            "sigmoid_gate: layout")
-    T, N = a.shape
+    """a * sigmoid(gate), element by element (fp32 inside) -> [T, N] contiguous.  gate [T, N]
+    rows with a contiguous last dim (may be a column slice of a wider row); a is [T, N] likewise,
+    or [H, T, V] with H * V == N -- the output of a batched product over heads -- whose heads are
+    concatenated here (no transposing copy)."""
+    if a.dim() == 3:
+        H, T, V = a.shape
+        if not use_hip(a, gate):
+            return (a.transpose(0, 1).reshape(T, H * V).float()
+                    * torch.sigmoid(gate.float())).to(a.dtype)
+        require(a.stride(2) == 1 and gate.shape == (T, H * V), "sigmoid_gate: head layout")
+        lda, a_sh, N = a.stride(1), a.stride(0), H * V
+    else:
+        if not use_hip(a, gate):
+            return (a.float() * torch.sigmoid(gate.float())).to(a.dtype)
+        require(a.dim() == 2 and a.shape == gate.shape and a.stride(1) == 1, "sigmoid_gate: layout")
+        T, N = a.shape
+        V, lda, a_sh = N, a.stride(0), 0
+    require(gate.stride(1) == 1 and a.dtype == gate.dtype and
+            a.dtype in (torch.bfloat16, torch.float32), "sigmoid_gate: layout")
     out = torch.empty(T, N, dtype=a.dtype, device=a.device)
-    check(lib().eia_sigmoid_gate(ptr(a), a.stride(0), ptr(gate), gate.stride(0), ptr(out),
+    check(lib().eia_sigmoid_gate(ptr(a), lda, a_sh, V, ptr(gate), gate.stride(0), ptr(out),
                                  out.stride(0), T, N, 1 if a.dtype == torch.bfloat16 else 0,
                                  stream(a)), "sigmoid_gate")
     return out

@@ -108,6 +108,16 @@ def case_sigmoid_gate(device, dtype):
         want = _np(a[:, a0:a0 + n]) * O.sigmoid(_np(gate[:, g0:g0 + n]))
         assert got.shape == (5, n) and got.is_contiguous()
         assert np.allclose(_np(got), want, atol=ktol(dtype), rtol=ktol(dtype))
+    # heads laid out [H, T, V] (a batched product's output) are concatenated on the way
+    for H, V in ((3, 10), (4, 16), (1, 7)):
+        a3 = (torch.randn(H, 5, V, generator=g) * 2).to(dtype).to(device)
+        got = activation.sigmoid_gate(a3, gate[:, 2:2 + H * V])
+        want = _np(a3).transpose(1, 0, 2).reshape(5, H * V) * O.sigmoid(_np(gate[:, 2:2 + H * V]))
+        assert got.shape == (5, H * V) and got.is_contiguous()
+        assert np.allclose(_np(got), want, atol=ktol(dtype), rtol=ktol(dtype))
+        got = activation.sigmoid_gate(a3, gate[:, 4:4 + H * V].contiguous())
+        want = _np(a3).transpose(1, 0, 2).reshape(5, H * V) * O.sigmoid(_np(gate[:, 4:4 + H * V]))
+        assert np.allclose(_np(got), want, atol=ktol(dtype), rtol=ktol(dtype))
 
 
 def case_frequencies():
