@@ -596,9 +596,24 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   // software pipeline (where the second operand set fits the register budget): block b + 1's
   // page lookup and K loads are in flight during block b's softmax and second product
   constexpr bool PIPE = NKV * P * ND <= 4;
+  // a wave with a single map and no head mixing has registers left to keep the next block's V^T
+  // operands in flight too, so no global load latency is exposed inside a block
+  constexpr bool VPIPE = PIPE && MW == 1 && !TALK;
   bf16x8 kf[NKV][P][2][ND], kn[PIPE ? NKV : 1][PIPE ? P : 1][2][PIPE ? ND : 1];
+  bf16x8 vn[VPIPE ? NKV : 1][VPIPE ? NDV : 1];
+  auto load_v = [&](int b, bf16x8 (&vv)[VPIPE ? NKV : 1][VPIPE ? NDV : 1]) {
+    const int key0 = (b < nsink ? b : wb0 + b - nsink) << 5;
+    const bf16_t* vp = vc + page_of(b, key0) * vpage + ((long)(hs / rep) * Dv + c) * bs +
+                       key0 % bs + dq;
+#pragma unroll
+    for (int t = 0; t < (VPIPE ? NDV : 1); ++t)
+      vv[0][t] = *reinterpret_cast<const bf16x8*>(vp + (long)(t < ndv ? t : 0) * 16 * bs);
+  };
   if constexpr (PIPE) {
     if (b_lo < b_hi) load_k(b_lo, kn);
+  }
+  if constexpr (VPIPE) {
+    if (b_lo < b_hi) load_v(b_lo, vn);
   }
   for (int b = b_lo; b < b_hi; ++b) {
     const int kb = b < nsink ? b : wb0 + b - nsink;                 // absolute 32-key block
@@ -647,14 +662,21 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
     if constexpr (PIPE) {
       if (b + 1 < b_hi) load_k(b + 1, kn);
     }
-    // the block's V^T operands are requested before the softmax arithmetic needs them
+    // the block's V^T operands are requested before the softmax arithmetic needs them (or were
+    // requested a block ago)
     bf16x8 vf[NKV][NDV];
+    if constexpr (VPIPE) {
 #pragma unroll
-    for (int j = 0; j < NKV; ++j) {
-      const bf16_t* vp = vc + page * vpage + ((long)((hs + j * HPK) / rep) * Dv + c) * bs + off + dq;
+      for (int t = 0; t < NDV; ++t) vf[0][t] = vn[0][t];
+      if (b + 1 < b_hi) load_v(b + 1, vn);
+    } else {
 #pragma unroll
-      for (int t = 0; t < NDV; ++t)
-        vf[j][t] = *reinterpret_cast<const bf16x8*>(vp + (long)(t < ndv ? t : 0) * 16 * bs);
+      for (int j = 0; j < NKV; ++j) {
+        const bf16_t* vp = vc + page * vpage + ((long)((hs + j * HPK) / rep) * Dv + c) * bs + off + dq;
+#pragma unroll
+        for (int t = 0; t < NDV; ++t)
+          vf[j][t] = *reinterpret_cast<const bf16x8*>(vp + (long)(t < ndv ? t : 0) * 16 * bs);
+      }
     }
     if constexpr (TALK) {
       // raw scores of every map through LDS: [buffer][map][tile][lane] f32x4
@@ -702,7 +724,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const float z = (e < 4 ? sc[m][0][e] : sc[m][1][e - 4]) + sbias[m];
-          const float p = vis[e] ? 1.0f / (1.0f + exp2f(-z * LOG2E)) : 0.f;
+          const float p = vis[e] ? __builtin_amdgcn_rcpf(1.0f + exp2f(-z * LOG2E)) : 0.f;
           const bf16_t hi = f2bf(p);
           ph[m][e] = hi;
           pl[m][e] = f2bf(p - bf2f(hi));
@@ -908,7 +930,9 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
                 2, part_acc, part_ml, wmode, bias};
   // raw-score buffers of the head-mixing form: two (one barrier per block) while they fit 48 KiB
   if (talk) a.raw_bufs = (size_t)2 * H * P * 128 * sizeof(f32x4) > 48 * 1024 ? 1 : 2;
-  const int hw = wa_mfma_hw(H, P, talk != nullptr);
+  // sigmoid weights: a wave takes two heads of one kv head where the grouping allows it, so the
+  // block's K / V^T operands are loaded once for both (the kernel is bound by those loads)
+  const int hw = (wmode == 1 && (H / G) % 2 == 0) ? 2 : wa_mfma_hw(H, P, talk != nullptr);
   const int waves_needed = H / hw;
   const int nwv = talk ? waves_needed : (waves_needed < 4 ? waves_needed : 4);
   const int gy = talk ? 1 : (waves_needed + nwv - 1) / nwv;
@@ -933,8 +957,14 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
     else WA_LAUNCH1(HWV, PV, TK, SH, 2, 4);                                                     \
   } while (0)
 #define WA_LAUNCH_SIG(NDX, NDVX)                                                                \
-  hipLaunchKernelGGL((window_attn_mfma_kernel<1, 1, false, true, NDX, NDVX, true>), grid, block, \
-                     lds, st, a)
+  do {                                                                                          \
+    if (hw == 2)                                                                                \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<2, 1, false, true, NDX, NDVX, true>), grid,   \
+                         block, lds, st, a);                                                    \
+    else                                                                                        \
+      hipLaunchKernelGGL((window_attn_mfma_kernel<1, 1, false, true, NDX, NDVX, true>), grid,   \
+                         block, lds, st, a);                                                    \
+  } while (0)
   // without head mixing the key width may be half the value width (a differential pair)
   const bool narrow_k = !talk && D <= 64 && Dv > 64;
   if (talk) {

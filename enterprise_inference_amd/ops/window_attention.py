@@ -8,8 +8,9 @@ map ``h*P + c`` reads key map ``(h // (H//G))*P + c`` and value head ``h // (H//
 the score of (query position i, key j) is ``(q.k) * mult[m] - slope[m]*(i-j)``, optionally mixed
 across maps by a matrix (``talk``), masked to ``j <= i and (i-j < window or j < keep)`` and
 soft-maxed -- or, with ``spec.weights`` 1, every visible key simply weighs
-``sigmoid(score + bias[m])`` and nothing is normalised over the keys.  ``spec.epilogue`` 0 multiplies the heads by ``sigmoid(gate)``; 1 combines a head's
-two maps as ``a1 - lam*a2``, divides by the root mean square over the head and scales.
+``sigmoid(score + bias[m])`` and nothing is normalised over the keys.  ``spec.epilogue`` 0
+multiplies the heads by ``sigmoid(gate)``; 1 combines a head's two maps as ``a1 - lam*a2``,
+divides by the root mean square over the head and scales.
 
 A step's rows are [decode rows (1 per sequence) | prefill chunks]; both parts read the cache
 after ``qk_norm_cache`` wrote this step's rows, so chunked prompts need no special path.
@@ -83,7 +84,9 @@ def decode_partitions(batch: int, spec: WindowSpec, cus: int = 256) -> int:
     forced = int(os.environ.get("EIA_WINDOW_DECODE_P", "0"))
     if forced > 0:
         return min(forced, 64)
-    wgs = max(1, batch) * (1 if spec.talk is not None else -(-spec.heads // 4))
+    # (sigmoid weights: a wave takes two heads where they share a kv head)
+    per_wave = 2 if (spec.weights == 1 and (spec.heads // spec.kv_heads) % 2 == 0) else 1
+    wgs = max(1, batch) * (1 if spec.talk is not None else -(-(spec.heads // per_wave) // 4))
     limit = 16
     if spec.window > 0:
         limit = max(1, min(16, ((spec.window + 31) // 32 + 1 + (spec.keep + 31) // 32) // 2))
