@@ -150,7 +150,8 @@ EIA_API int eia_splitk_act_and_mul(const float* part, int sk, int T, int F, void
 // xIELU with two learned numbers (p, q) read from device memory (a weight reload needs no new
 // launch arguments):  z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z)
 // + z/2.  fp32 inside.  The input is a stored row [T, F] (type T, row stride ldx) or the fp32
-// split-K partials [sk, T, F] of the GEMM that produced it, summed here (F % 4 == 0 then).
+// split-K partials [sk, T, ldp] of the GEMM that produced it (the F columns from the pointer on;
+// a fused projection's row is wider than F), summed here (F, ldp % 4 == 0 then).
 EIA_DEV float softplus_f(float z) { return fmaxf(z, 0.f) + log1pf(expf(-fabsf(z))); }
 EIA_DEV float xielu_f(float z, float ap, float aq) {
   return z > 0.f ? ap * z * z + 0.5f * z : aq * (expm1f(z) - z) + 0.5f * z;
@@ -171,15 +172,15 @@ template <> EIA_DEV void act_st4<float>(float* p, f32x4 v) { *reinterpret_cast<f
 
 template <typename T>
 __global__ void __launch_bounds__(256)
-xielu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ part, int sk,
+xielu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ part, int sk, long ldp,
              const T* __restrict__ pq, T* __restrict__ out, long ldo, int rows, int F, int vec) {
   const float ap = softplus_f(ld_f32<T>(pq, 0)), aq = 0.5f + softplus_f(ld_f32<T>(pq, 1));
   if (part) {
     const long idx = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (idx >= (long)rows * F) return;
     const int row = idx / F, col = idx % F;
-    const long slab = (long)rows * F;
-    const float* p = part + idx;
+    const long slab = (long)rows * ldp;              // rows of the partials are ldp wide
+    const float* p = part + (long)row * ldp + col;
     f32x4 v = *reinterpret_cast<const f32x4*>(p);
     for (int z = 1; z < sk; ++z) v += *reinterpret_cast<const f32x4*>(p + z * slab);
     if (vec) {
@@ -206,10 +207,10 @@ xielu_kernel(const T* __restrict__ x, long ldx, const float* __restrict__ part, 
   st_f32<T>(out + (long)row * ldo, col, xielu_f(ld_f32<T>(x + (long)row * ldx, col), ap, aq));
 }
 
-EIA_API int eia_xielu(const void* x, long ldx, const float* part, int sk, const void* pq, void* out,
-                      long ldo, int rows, int F, int is_bf16, hipStream_t st) {
+EIA_API int eia_xielu(const void* x, long ldx, const float* part, int sk, long ldp, const void* pq,
+                      void* out, long ldo, int rows, int F, int is_bf16, hipStream_t st) {
   if (rows < 0 || F < 1 || !pq || !out || (x == nullptr) == (part == nullptr) ||
-      (part && (sk < 1 || F % 4)))
+      (part && (sk < 1 || F % 4 || ldp % 4 || ldp < F || reinterpret_cast<uintptr_t>(part) % 16)))
     return EIA_BAD_SHAPE;
   if (rows == 0) return EIA_OK;
   const int esz = is_bf16 ? 2 : 4;
@@ -219,10 +220,10 @@ EIA_API int eia_xielu(const void* x, long ldx, const float* part, int sk, const 
   dim3 grid((unsigned)((n + 255) / 256)), block(256);
   if (is_bf16)
     hipLaunchKernelGGL(xielu_kernel<bf16_t>, grid, block, 0, st, (const bf16_t*)x, ldx, part, sk,
-                       (const bf16_t*)pq, (bf16_t*)out, ldo, rows, F, vec);
+                       ldp, (const bf16_t*)pq, (bf16_t*)out, ldo, rows, F, vec);
   else
     hipLaunchKernelGGL(xielu_kernel<float>, grid, block, 0, st, (const float*)x, ldx, part, sk,
-                       (const float*)pq, (float*)out, ldo, rows, F, vec);
+                       ldp, (const float*)pq, (float*)out, ldo, rows, F, vec);
   EIA_LAUNCH_CHECK();
 }
 

@@ -32,21 +32,6 @@ EIA_DEV float lat_rotated(const T* src, int d, int rot_dims, bool half, float am
   return second ? (w * cs + u * sn) : (u * cs - w * sn);
 }
 
-// Entries dd0 .. dd0 + 7 of a rotary query part after the rotation (entries past rot_dims pass
-// unchanged).  Not inlined: one copy of the sine / cosine code per kernel.
-__device__ __attribute__((noinline)) bf16x8
-lat_rot_chunk(const bf16_t* qr, int dd0, int rot_dims, bool half, float amp, float pos,
-              const float* __restrict__ inv_freq) {
-  bf16x8 v;
-#pragma unroll 1
-  for (int e = 0; e < 8; ++e) {
-    const int dd = dd0 + e;
-    v[e] = f2bf(dd < rot_dims ? lat_rotated<bf16_t>(qr, dd, rot_dims, half, amp, pos, inv_freq)
-                              : bf2f(qr[dd]));
-  }
-  return v;
-}
-
 // ------------------------------------------------------------------------------------------ prep
 // fused [T, ld]: columns [q_off, q_off+q_rank) query latent, [c_off, c_off+R) KV latent,
 // [kr_off, kr_off+rd) shared rotary key part.  q_rank == 0: no query latent; cache == nullptr:
@@ -391,6 +376,11 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
     ntok = 1;
   }
   if (ntok <= 0 || (a.seq_lens && a.seq_lens[seq] <= 0)) return;
+  {   // a partition beyond the ones this row's context uses has nothing to do (whole workgroup)
+    const int kmax0 = a.positions[row0 + ntok - 1] + 1;
+    const int kmin0 = a.window > 0 ? (max(0, a.positions[row0] - a.window + 1) & ~31) : 0;
+    if ((int)blockIdx.z >= lat_parts(a.nparts, kmin0, kmax0)) return;
+  }
   const int h0 = blockIdx.y * a.HB;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = lane & 15, g = lane >> 4;
@@ -403,13 +393,41 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
   const bool row_ok = t < ntok && h < a.H && m < a.QB * a.HB;
   const long row = row0 + (row_ok ? t : 0);
   const int qpos = row_ok ? a.positions[row] : -1;
+  // the rotary query parts of the workgroup's rows, rotated once into LDS: a thread takes whole
+  // pairs (one sine / cosine each, independent loads), not the entries of its own operand
+  bf16_t* qrs = vt + nc * 16 * LDV;                        // [rows][rd]
+  {
+    constexpr int NROWS = SPLITV ? 16 : NW * 16;
+    const bf16_t* qrb = static_cast<const bf16_t*>(a.qr);
+    const int hp = a.rot_dims >> 1, npass = a.rd - a.rot_dims;
+    for (int e = tid; e < NROWS * hp; e += NT) {
+      const int mm = e / hp, i = e - mm * hp;
+      const int tt = mm / a.HB, hh = h0 + (mm - tt * a.HB);
+      if (tt < ntok && hh < a.H && mm < a.QB * a.HB) {
+        const bf16_t* src = qrb + (long)(row0 + tt) * a.qr_st + (long)hh * a.qr_sh;
+        const int ia = a.rot_half ? i : 2 * i, ib = a.rot_half ? i + hp : 2 * i + 1;
+        const float u = bf2f(src[ia]), w = bf2f(src[ib]);
+        float sn, cs;
+        sincosf((float)a.positions[row0 + tt] * a.inv_freq[i], &sn, &cs);
+        sn *= a.rot_amp;
+        cs *= a.rot_amp;
+        qrs[mm * a.rd + ia] = f2bf(u * cs - w * sn);
+        qrs[mm * a.rd + ib] = f2bf(w * cs + u * sn);
+      }
+    }
+    for (int e = tid; e < NROWS * npass; e += NT) {        // entries past rot_dims pass unchanged
+      const int mm = e / npass, d = a.rot_dims + (e - mm * npass);
+      const int tt = mm / a.HB, hh = h0 + (mm - tt * a.HB);
+      if (tt < ntok && hh < a.H && mm < a.QB * a.HB)
+        qrs[mm * a.rd + d] = qrb[(long)(row0 + tt) * a.qr_st + (long)hh * a.qr_sh + d];
+    }
+    __syncthreads();
+  }
   bf16x8 qf[NKMAX];
   {
     const bf16_t* qa = static_cast<const bf16_t*>(a.qa) + row * a.qa_st + (long)h * a.qa_sh;
-    const bf16_t* qr = static_cast<const bf16_t*>(a.qr) + row * a.qr_st + (long)h * a.qr_sh;
-    // R % 8 == 0: a lane's 8-entry chunk lies wholly in the absorbed part (one 16-byte load when
-    // the rows are aligned) or wholly in the rotary part (rotated by a called, rolled helper:
-    // the sine / cosine code exists once, not once per entry of the unrolled operand)
+    // R % 8 == 0 and rd % 8 == 0: a lane's 8-entry chunk lies wholly in the absorbed part (one
+    // 16-byte load when the rows are aligned) or wholly in the rotary part (one LDS read)
     const bool qvec = ((reinterpret_cast<uintptr_t>(a.qa) | (uintptr_t)(a.qa_st * 2) |
                         (uintptr_t)(a.qa_sh * 2)) & 15) == 0;
 #pragma unroll
@@ -418,8 +436,7 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
       bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
       if (row_ok && s < nk && d0 < Dk) {
         if (d0 >= a.R) {
-          v = lat_rot_chunk(qr, d0 - a.R, a.rot_dims, a.rot_half != 0, a.rot_amp, (float)qpos,
-                            a.inv_freq);
+          v = *reinterpret_cast<const bf16x8*>(qrs + m * a.rd + (d0 - a.R));
         } else if (qvec) {
           v = *reinterpret_cast<const bf16x8*>(qa + d0);
         } else {
@@ -450,7 +467,6 @@ latent_attn_mfma_kernel(LatentAttnArgs a) {
     k_begin = kmin + (min((int)blockIdx.z * per, units) << 5);
     k_end = min(kmax, kmin + (((int)blockIdx.z + 1) * per << 5));
   }
-  if ((int)blockIdx.z >= np) return;                       // (whole workgroup)
   const int wlo = a.window > 0 ? qpos - a.window + 1 : 0;   // first key this lane's row sees
   const int cpr = Dkp >> 3;                                // 16-byte chunks per (padded) key row
   const int nchunk = 32 * cpr;
@@ -667,7 +683,8 @@ EIA_API int eia_latent_attn_mfma(const void* qa, long qa_st, long qa_sh, const v
     return EIA_BAD_SHAPE;
   const int nk = (Dk + 31) / 32, Dkp = nk * 32, nc = (R + 15) / 16;
   const int ldk = ((Dkp / 8) & 1) ? Dkp : Dkp + 8;       // odd number of 16-byte units per row
-  const size_t lds = ((size_t)32 * ldk + (size_t)nc * 16 * 40) * 2;
+  // K tile, V^T tile, and the rotated rotary query parts of up to 64 rows
+  const size_t lds = ((size_t)32 * ldk + (size_t)nc * 16 * 40 + (size_t)64 * rd) * 2;
   LatentAttnArgs a{qa, qa_st, qa_sh, qr, qr_st, qr_sh, inv_freq, rot_dims, cache, cache_row,
                    block_table, bt_stride, seq_lens, cu_q, work, n_items, positions, gate, gate_st,
                    out, out_st, out_sh, scale, H, R, rd, bs, QB, HB, 32, ldk, window, sink, rot_half,

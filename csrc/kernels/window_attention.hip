@@ -131,14 +131,16 @@ qk_rope_cache_kernel(const T* __restrict__ fused, long ld, const float* __restri
                      const T* __restrict__ kw, const float* __restrict__ inv_freq, int rot_dims,
                      int half, float amp, const int* __restrict__ positions, T* __restrict__ q_out,
                      long ldq, T* __restrict__ kc, T* __restrict__ vc,
-                     const int* __restrict__ slots, int bs, float eps) {
+                     const int* __restrict__ slots, int bs, float eps, int nsum) {
   __shared__ float scratch[4];
   const long t = blockIdx.x;
   const long slot = slots ? (long)slots[t] : -1;
   extern __shared__ float rsum[];                   // [ld] when the row arrives as partials
   const int hd = rot_dims >> 1;
   // the token's cos / sin (times amp), once per pair index, behind the summed row
-  float* cs_t = rsum + (part ? ld : 0);             // [hd] cos, then [hd] sin
+  // (nsum: the row's first columns that hold q, k and v, a multiple of 4; a fused projection's
+  // row may go on with other consumers' columns)
+  float* cs_t = rsum + (part ? nsum : 0);           // [hd] cos, then [hd] sin
   for (int i = threadIdx.x; i < hd; i += blockDim.x) {
     float sn, cs;
     sincosf((float)positions[t] * inv_freq[i], &sn, &cs);
@@ -146,7 +148,7 @@ qk_rope_cache_kernel(const T* __restrict__ fused, long ld, const float* __restri
     cs_t[hd + i] = sn * amp;
   }
   if (part) {
-    for (int c = 4 * threadIdx.x; c < (int)ld; c += 4 * blockDim.x) {
+    for (int c = 4 * threadIdx.x; c < nsum; c += 4 * blockDim.x) {
       f32x4 v = {0.f, 0.f, 0.f, 0.f};
       if (bias) v = f32x4{ld_f32<T>(bias, c), ld_f32<T>(bias, c + 1), ld_f32<T>(bias, c + 2),
                           ld_f32<T>(bias, c + 3)};
@@ -207,20 +209,25 @@ EIA_API int eia_qk_rope_cache(const void* fused, long ld, const float* part, int
     return EIA_BAD_SHAPE;
   if (T == 0) return EIA_OK;
   const long ps = (long)T * ld;
-  const size_t lds = (part ? sizeof(float) * ld : 0) + sizeof(float) * rot_dims;
+  int nsum = q_off + MQ * D;
+  if (k_off + MK * D > nsum) nsum = k_off + MK * D;
+  if (v_off + VW > nsum) nsum = v_off + VW;
+  nsum = (nsum + 3) & ~3;                           // (<= ld: ld % 4 == 0)
+  if (part && nsum > ld) return EIA_BAD_SHAPE;
+  const size_t lds = (part ? sizeof(float) * nsum : 0) + sizeof(float) * rot_dims;
   if (lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (is_bf16)
     hipLaunchKernelGGL((qk_rope_cache_kernel<bf16_t>), dim3(T), dim3(256), lds, st,
                        (const bf16_t*)fused, ld, part, sk, ps, (const bf16_t*)bias, q_off, k_off,
                        v_off, MQ, MK, D, VW, (const bf16_t*)qw, (const bf16_t*)kw, inv_freq,
                        rot_dims, half, amp, positions, (bf16_t*)q_out, ldq, (bf16_t*)kc,
-                       (bf16_t*)vc, slots, bs, eps);
+                       (bf16_t*)vc, slots, bs, eps, nsum);
   else
     hipLaunchKernelGGL((qk_rope_cache_kernel<float>), dim3(T), dim3(256), lds, st,
                        (const float*)fused, ld, part, sk, ps, (const float*)bias, q_off, k_off,
                        v_off, MQ, MK, D, VW, (const float*)qw, (const float*)kw, inv_freq, rot_dims,
                        half, amp, positions, (float*)q_out, ldq, (float*)kc, (float*)vc, slots, bs,
-                       eps);
+                       eps, nsum);
   EIA_LAUNCH_CHECK();
 }
 

@@ -88,7 +88,7 @@ _SIGNATURES = {
     "eia_qk_rope_cache": [P, L, P, I, P, I, I, I, I, I, I, I, P, P, P, I, I, F, IP, P, L, P, P, IP,
                           I, F, I, I, S],
     "eia_add_rms": [P, L, P, I, P, P, L, P, I, P, P, P, P, L, F, I, I, I, S],
-    "eia_xielu": [P, L, P, I, P, P, L, I, I, I, S],
+    "eia_xielu": [P, L, P, I, L, P, P, L, I, I, I, S],
     "eia_sigmoid_gate": [P, L, L, I, P, L, P, L, I, I, I, S],
     "eia_window_attn_mfma_ok": [I, I, I, I, I, I, I],
     "eia_ar_alloc": [P, L],

@@ -19,8 +19,10 @@ scaling{factor, original, fast, slow}}}, mlp{kind: dense, ff} | null}.  Checkpoi
 head, final.norm, l<i>.norm1, l<i>.mix.*, l<i>.mlp.up|down|act.
 
 Residual stream, norms, angles, scores, attention weights and gates are fp32 whatever the
-activation dtype; with dtype float32 the matrix products are fp32 too.  A layer boundary (both
-residual adds and the next layer's input norm) is one launch (ops/norm.py residual_rms_step).
+activation dtype; with dtype float32 the matrix products are fp32 too.  Both sublayers read the
+same h, so the feed-forward's up-projection rides in the mixer's fused input projection (one
+GEMM per layer input), and a layer boundary (both residual adds and the next layer's input
+norm) is one launch (ops/norm.py residual_rms_step).
 """
 
 from __future__ import annotations
@@ -52,6 +54,12 @@ class GapidraLayer(nn.Module):
         super().__init__()
         m = spec["mixer"]
         self.kind = spec["type"]
+        mlp = spec.get("mlp")
+        if mlp is not None and mlp.get("kind", "dense") != "dense":
+            raise ValueError(f"unknown Gapidra feed-forward kind {mlp.get('kind')!r}")
+        # both sublayers read the same h: the feed-forward's up-projection rides in the mixer's
+        # fused input projection (one GEMM per layer input)
+        ff = int(mlp["ff"]) if mlp is not None else 0
         window = int((m.get("mask") or {}).get("size", 0))
         rot = m.get("rot") or {}
         if self.kind == "latent_attention":
@@ -60,30 +68,28 @@ class GapidraLayer(nn.Module):
                 width, m["heads"], m["dim"], rd, m.get("vdim", m["dim"]), m["kv_rank"], 0,
                 m["scale"], int(rot.get("dims", rd)), float(rot.get("base", 10000.0)), eps,
                 own_kv=True, dtype=dtype, device=device, gate="element", window=window, sink=True,
-                rot_half=True, rot_scaling=rot.get("scaling"), defer_out=True)
+                rot_half=True, rot_scaling=rot.get("scaling"), defer_out=True, extra_rows=ff)
         elif self.kind == "attention":
             self.mix = SigmoidWindowAttentionMixer(
                 width, m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"]),
                 m["scale"], window, int(rot.get("dims", 0)), float(rot.get("base", 10000.0)),
-                rot.get("scaling"), eps, dtype, device)
+                rot.get("scaling"), eps, dtype, device, extra_rows=ff)
         else:
             raise ValueError(f"unknown Gapidra layer type {self.kind!r}")
         self.norm1 = _norm_weight(width, dtype, device)
         self.eps = eps
-        mlp = spec.get("mlp")
         self.mlp = None
         if mlp is not None:
-            if mlp.get("kind", "dense") != "dense":
-                raise ValueError(f"unknown Gapidra feed-forward kind {mlp.get('kind')!r}")
-            self.mlp = UngatedMLP(width, mlp["ff"], dtype, device, act="xielu", defer=True)
+            self.mlp = UngatedMLP(width, ff, dtype, device, act="xielu", defer=True, own_up=False)
 
     def forward(self, x: torch.Tensor, h: torch.Tensor, md: AttentionMetadata, cache,
                 w_next: Optional[torch.Tensor]):
         """x: fp32 residual [T, width], updated in place; h = norm1(x) in the activation dtype.
         Returns the next layer's input norm of the new x, or None when ``w_next`` is None."""
-        y = self.mix(h, md, cache)
-        f = self.mlp(h) if self.mlp is not None else None
-        return norm_ops.residual_rms_step(x, self.eps, (y, f), w_next)
+        if self.mlp is None:
+            return norm_ops.residual_rms_step(x, self.eps, (self.mix(h, md, cache),), w_next)
+        y, up = self.mix(h, md, cache, want_extra=True)
+        return norm_ops.residual_rms_step(x, self.eps, (y, self.mlp(None, pre=up)), w_next)
 
 
 class GapidraForCausalLM(nn.Module):
@@ -176,7 +182,7 @@ class GapidraForCausalLM(nn.Module):
                "dkv.norm": ("kv_norm", None)}
     _ATTN = {"q": ("proj", "q"), "k": ("proj", "k"), "v": ("proj", "v"),
              "q.norm": ("q_norm", None), "k.norm": ("k_norm", None)}
-    _MLP = {"up": "up.weight", "down": "down.weight", "act": "act"}
+    _MLP = {"down": "down.weight", "act": "act"}
 
     def _target(self, name: str):
         """checkpoint name -> (parameter name, shard id)."""
@@ -195,6 +201,9 @@ class GapidraForCausalLM(nn.Module):
             table = self._LATENT if self.layers[i].kind == "latent_attention" else self._ATTN
             p, sid = table.get(rest[4:], (rest[4:], None))
             return pre + "mix." + p, sid
+        if rest == "mlp.up":              # rows of the mixer's fused input projection
+            fused = "down" if self.layers[i].kind == "latent_attention" else "proj"
+            return pre + "mix." + fused, "x"
         if rest.startswith("mlp.") and rest[4:] in self._MLP:
             return pre + "mlp." + self._MLP[rest[4:]], None
         return None, None
@@ -232,11 +241,14 @@ class GapidraForCausalLM(nn.Module):
                 p.data.copy_(torch.randn(p.shape, generator=g, device=p.device) * 0.3)
             elif leaf in ("proj", "down") and name.endswith(("mix.proj", "mix.down")):
                 mix = self.get_submodule(name.rsplit(".", 1)[0])
-                rows = (sum(n for _, n in mix.offsets.values()) if leaf == "proj"
-                        else mix.q_rows + mix.kv_rows + mix.gate_rows)
-                p.data.zero_()
-                p.data[:rows].copy_(torch.randn((rows, p.shape[1]), generator=g, device=p.device,
-                                                dtype=torch.float32) * p.shape[-1] ** -0.5)
+                spans = (list(mix.offsets.values()) if leaf == "proj" else
+                         [(0, mix.q_rows + mix.kv_rows + mix.gate_rows),
+                          (mix.extra_off, mix.extra_rows)])
+                p.data.zero_()                      # pad rows stay zero
+                for off, rows in spans:
+                    p.data[off:off + rows].copy_(
+                        torch.randn((rows, p.shape[1]), generator=g, device=p.device,
+                                    dtype=torch.float32) * p.shape[-1] ** -0.5)
             else:
                 p.data.copy_(torch.randn(p.shape, generator=g, device=p.device,
                                          dtype=torch.float32) * p.shape[-1] ** -0.5)

@@ -76,13 +76,16 @@ class LatentAttentionMixer(nn.Module):
     ``sink``: a learned per-head term exp(sink_h) in the softmax denominator.  ``rot_half``:
     rotation pairs (i, i + dims/2) instead of (2i, 2i+1); ``rot_scaling``: frequency
     interpolation (ops/rotary.py rotary_frequencies).  ``defer_out``: hand the output
-    projection's split-K partials to the caller's boundary step."""
+    projection's split-K partials to the caller's boundary step.  ``extra_rows``: that many more
+    rows ride in the fused input projection (shard "x": another consumer of the same layer
+    input, e.g. a feed-forward that runs beside the mixer); ``forward(..., want_extra=True)``
+    then returns (output, their columns)."""
 
     def __init__(self, width: int, heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int,
                  q_rank: int, scale: float, rot_dims: int, rot_base: float, eps: float,
                  own_kv: bool, dtype, device, *, gate: str = "head", window: int = 0,
                  sink: bool = False, rot_half: bool = False, rot_scaling=None,
-                 defer_out: bool = False):
+                 defer_out: bool = False, extra_rows: int = 0):
         super().__init__()
         if pstate.tp_size() != 1:
             raise NotImplementedError("latent attention runs on one rank (no head sharding yet)")
@@ -103,8 +106,11 @@ class LatentAttentionMixer(nn.Module):
         # (rows padded with zeros to a multiple of 64: decode-sized batches then run the
         # weight-streaming GEMM, whose row tiles need it; the pad columns are never read)
         n = self.q_rows + self.kv_rows + self.gate_rows
+        self.extra_rows = int(extra_rows)
+        self.extra_off = -(-n // 8) * 8 if extra_rows else n      # (16-byte aligned columns)
+        n = self.extra_off + self.extra_rows
         self.down = _param((-(-n // 64) * 64, width), dtype, device)
-        self.down.data[n:].zero_()
+        self.down.data.zero_()
         self.down.weight_loader = self._load_down
         self.q_norm = _plain((q_rank,), dtype, device) if q_rank else None
         self.kv_norm = _plain((kv_rank,), dtype, device) if own_kv else None
@@ -127,13 +133,16 @@ class LatentAttentionMixer(nn.Module):
             self.sink_f32.copy_(self.sink.float())
 
     def _load_down(self, param, loaded, shard_id=None):
-        off = {"dq": 0, "q": 0, "dkv": self.q_rows, "g": self.q_rows + self.kv_rows}[shard_id]
-        rows = {"dq": self.q_rows, "q": self.q_rows, "dkv": self.kv_rows, "g": self.gate_rows}[shard_id]
+        off = {"dq": 0, "q": 0, "dkv": self.q_rows, "g": self.q_rows + self.kv_rows,
+               "x": self.extra_off}[shard_id]
+        rows = {"dq": self.q_rows, "q": self.q_rows, "dkv": self.kv_rows, "g": self.gate_rows,
+                "x": self.extra_rows}[shard_id]
         if loaded.shape[0] != rows or param.data[off:off + rows].shape != loaded.shape:
             raise ValueError(f"latent attention {shard_id}: shape {tuple(loaded.shape)}")
         param.data[off:off + rows].copy_(loaded)
 
-    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: LatentKVCache):
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: LatentKVCache,
+                want_extra: bool = False):
         T = xb.shape[0]
         H, D, rd, R = self.heads, self.dim, self.rot_dim, self.kv_rank
         fused = gemm.linear(xb, self.down)
@@ -159,7 +168,10 @@ class LatentAttentionMixer(nn.Module):
             o = act_ops.sigmoid_gate(o, fused[:, g0:g0 + self.gate_rows])
         else:
             o = o.transpose(0, 1).reshape(T, H * self.vdim)
-        return gemm.linear(o, self.o, defer_reduce=self.defer_out)
+        y = gemm.linear(o, self.o, defer_reduce=self.defer_out)
+        if want_extra:
+            return y, fused[:, self.extra_off:self.extra_off + self.extra_rows]
+        return y
 
 
 class WKVMixer(nn.Module):
@@ -255,10 +267,12 @@ class _WindowMixerBase(nn.Module):
         self.scale, self.window, self.keep, self.eps = float(scale), int(window), int(keep), float(eps)
         self.offsets, n = {}, 0
         for name, rows in parts:
+            if name == "x":                  # another consumer's rows: 16-byte aligned columns
+                n = -(-n // 8) * 8
             self.offsets[name] = (n, rows)
             n += rows
         self.proj = _param((_pad64(n), width), dtype, device)
-        self.proj.data[n:].zero_()
+        self.proj.data.zero_()
         self.proj.weight_loader = self._load_part
         self.proj_bias = None
         if bias:
@@ -376,16 +390,20 @@ class SigmoidWindowAttentionMixer(_WindowMixerBase):
     key projection are each RMS-normed as ONE vector (weights of their full size) before the
     first ``rot_dims`` entries of every head turn by the position (pairs (2i, 2i+1), or
     (i, i + rot_dims/2) with ``rot_half``; ``rot_scaling`` as in ops/rotary.py
-    rotary_frequencies).  No biases, no gate."""
+    rotary_frequencies).  No biases, no gate.  ``extra_rows``: that many more rows ride in the
+    fused input projection (part "x": another consumer of the same layer input);
+    ``forward(..., want_extra=True)`` then returns (output, their columns)."""
 
     def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
                  window: int, rot_dims: int, rot_base: float, rot_scaling, eps: float, dtype,
-                 device, rot_half: bool = False):
+                 device, rot_half: bool = False, extra_rows: int = 0):
         super().__init__()
         if rot_dims > dim or rot_dims % 2:
             raise ValueError("rot.dims must be even and at most dim")
-        self._setup(width, heads, kv_heads, dim, vdim, scale, window, 0, eps,
-                    [("q", heads * dim), ("k", kv_heads * dim), ("v", kv_heads * vdim)], False,
+        parts = [("q", heads * dim), ("k", kv_heads * dim), ("v", kv_heads * vdim)]
+        if extra_rows:
+            parts.append(("x", int(extra_rows)))
+        self._setup(width, heads, kv_heads, dim, vdim, scale, window, 0, eps, parts, False,
                     dtype, device, norm_sizes=(heads * dim, kv_heads * dim))
         self.rot_dims, self.rot_half = int(rot_dims), rot_half
         self.inv_freq, self.rot_amp = rot_ops.rotary_frequencies(rot_dims, rot_base, rot_scaling,
@@ -397,7 +415,8 @@ class SigmoidWindowAttentionMixer(_WindowMixerBase):
     def refresh(self) -> None:
         self.spec.bias.copy_(self.pb.float())
 
-    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows):
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows,
+                want_extra: bool = False):
         fused = gemm.linear(xb, self.proj, None, defer_reduce=True)
         q = win_ops.qk_rope_cache(fused, self.offsets["q"][0], self.offsets["k"][0],
                                   self.offsets["v"][0], self.heads, self.kv_heads, self.dim,
@@ -406,4 +425,7 @@ class SigmoidWindowAttentionMixer(_WindowMixerBase):
                                   md.positions, cache.k, cache.v, md.slot_mapping, self.eps)
         a = win_ops.window_attention(q, cache.k, cache.v, md, self.spec, None)
         # may return gemm.SplitK: the layer's boundary step reduces it
-        return gemm.linear(a, self.o, defer_reduce=True)
+        y = gemm.linear(a, self.o, defer_reduce=True)
+        if want_extra:
+            return y, gemm.columns(fused, *self.offsets["x"])
+        return y

@@ -202,25 +202,34 @@ class UngatedMLP(nn.Module):
     (softplus(p) z^2 + z/2 above zero, (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2 below, with
     the layer's two learned numbers (p, q) in the parameter ``act``).  With ``defer`` the
     decode-sized products hand their split-K partial sums on: the up-projection's to the
-    activation kernel, the down-projection's to the caller's boundary step."""
+    activation kernel, the down-projection's to the caller's boundary step.  ``own_up=False``:
+    the up-projection's rows live in another module's fused projection of the same input, and
+    ``forward(None, pre=...)`` takes its output (a tensor or split-K partial columns)."""
 
     def __init__(self, hidden: int, inter: int, dtype, device, act: str = "relu2",
-                 defer: bool = False):
+                 defer: bool = False, own_up: bool = True):
         super().__init__()
         if act not in ("relu2", "xielu"):
             raise ValueError(f"UngatedMLP: unknown activation {act!r}")
-        self.up = ReplicatedLinear(hidden, inter, dtype=dtype, device=device)
+        self.up = ReplicatedLinear(hidden, inter, dtype=dtype, device=device) if own_up else None
         self.down = ReplicatedLinear(inter, hidden, dtype=dtype, device=device)
         self.kind, self.defer = act, defer
         if act == "xielu":
             self.act = _param((2,), dtype, device)
             self.act.weight_loader = lambda p, t, sid=None: p.data.copy_(t.reshape(2))
 
-    def forward(self, x):
+    def forward(self, x, pre=None):
         from ..ops import activation, gemm
+        from ..ops.gemm import SplitK, SplitKSlice
+        if pre is None:
+            pre = gemm.linear(x, self.up.weight, defer_reduce=self.defer and self.kind == "xielu")
         if self.kind == "relu2":
-            return self.down(activation.relu2(self.up(x)))
-        z = activation.xielu(gemm.linear(x, self.up.weight, defer_reduce=self.defer), self.act)
+            if isinstance(pre, SplitKSlice):
+                pre = pre.dense(self.down.weight.dtype)
+            elif isinstance(pre, SplitK):
+                pre = pre.materialize()
+            return self.down(activation.relu2(pre.contiguous()))
+        z = activation.xielu(pre, self.act)
         return gemm.linear(z, self.down.weight, defer_reduce=self.defer)
 
 

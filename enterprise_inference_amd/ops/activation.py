@@ -68,9 +68,21 @@ def relu2(x: torch.Tensor) -> torch.Tensor:
 def xielu(x, pq: torch.Tensor) -> torch.Tensor:
     """xIELU with the two learned numbers ``pq`` = (p, q) read from device memory:
     z > 0: softplus(p) z^2 + z/2;  z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2, evaluated
-    in fp32.  x [T, F] in the activation dtype, or a ``gemm.SplitK`` (fp32 partial sums of the
-    up-projection, summed here) -> [T, F] in pq's dtype."""
-    from .gemm import SplitK
+    in fp32.  x [T, F] in the activation dtype (rows may be a column slice of a wider row), or a
+    ``gemm.SplitK`` / ``gemm.SplitKSlice`` (fp32 partial sums of the up-projection, or of a fused
+    projection that holds it, summed here) -> [T, F] in pq's dtype."""
+    from .gemm import SplitK, SplitKSlice
+    if isinstance(x, SplitKSlice):          # some columns of a fused projection's partials
+        src = x.src
+        if src.part.is_cuda and src.bias is None and x.n % 4 == 0 and x.off % 4 == 0 and \
+                src.N % 4 == 0 and src.part.is_contiguous() and pq.dtype in (torch.bfloat16,
+                                                                             torch.float32):
+            out = torch.empty(src.M, x.n, dtype=pq.dtype, device=pq.device)
+            check(lib().eia_xielu(None, 0, src.part.data_ptr() + 4 * x.off, src.sk, src.N, ptr(pq),
+                                  ptr(out), out.stride(0), src.M, x.n,
+                                  1 if pq.dtype == torch.bfloat16 else 0, stream(out)), "xielu")
+            return out
+        x = x.dense(pq.dtype)
     split = isinstance(x, SplitK)
     if split and not (x.part.is_cuda and x.bias is None and x.N % 4 == 0 and x.part.is_contiguous()):
         x = (x.part.sum(0) + (x.bias.float() if x.bias is not None else 0.0)).to(pq.dtype)
@@ -88,13 +100,13 @@ def xielu(x, pq: torch.Tensor) -> torch.Tensor:
     if split:
         T, F = x.M, x.N
         out = torch.empty(T, F, dtype=dt, device=pq.device)
-        check(lib().eia_xielu(None, 0, ptr(x.part), x.sk, ptr(pq), ptr(out), out.stride(0), T, F,
+        check(lib().eia_xielu(None, 0, ptr(x.part), x.sk, F, ptr(pq), ptr(out), out.stride(0), T, F,
                               1 if dt == torch.bfloat16 else 0, stream(out)), "xielu")
         return out
     require(x.dim() == 2 and x.stride(1) == 1 and x.dtype == dt, "xielu: row layout")
     T, F = x.shape
     out = torch.empty(T, F, dtype=dt, device=x.device)
-    check(lib().eia_xielu(ptr(x), x.stride(0), None, 0, ptr(pq), ptr(out), out.stride(0), T, F,
+    check(lib().eia_xielu(ptr(x), x.stride(0), None, 0, 0, ptr(pq), ptr(out), out.stride(0), T, F,
                           1 if dt == torch.bfloat16 else 0, stream(out)), "xielu")
     return out
 

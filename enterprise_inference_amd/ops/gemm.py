@@ -396,6 +396,28 @@ class SplitK:
         return o
 
 
+class SplitKSlice:
+    """Columns [off, off + n) of a ``SplitK``: one consumer of a GEMM whose output row holds the
+    inputs of several (a fused projection).  ``off`` is a multiple of 4 for the fused reducers."""
+
+    __slots__ = ("src", "off", "n")
+
+    def __init__(self, src: SplitK, off: int, n: int):
+        self.src, self.off, self.n = src, off, n
+
+    def dense(self, dtype) -> torch.Tensor:
+        s = self.src
+        r = s.part[:, :, self.off:self.off + self.n].sum(0)
+        if s.bias is not None:
+            r = r + s.bias[self.off:self.off + self.n].float()
+        return r.to(dtype)
+
+
+def columns(y, off: int, n: int):
+    """Columns [off, off + n) of a GEMM output that is a tensor or a ``SplitK``."""
+    return SplitKSlice(y, off, n) if isinstance(y, SplitK) else y[:, off:off + n]
+
+
 def skinny(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None,
            defer_reduce: bool = False, cfg: Optional[int] = None, sk: Optional[int] = None):
     """x [M, K] @ w[N, K]^T on the skinny kernel. Returns a tensor or a SplitK."""

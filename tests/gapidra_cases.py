@@ -95,6 +95,14 @@ def case_xielu(device, dtype):
         # (a width the kernel does not sum itself is rounded to the dtype before the activation)
         loose = 6e-2 if (dtype != torch.float32 and F % 4) else ktol(dtype)
         assert np.allclose(_np(got), want, atol=loose, rtol=loose), (F, p, q, "partials")
+        # the same columns inside the wider row of a fused projection's partial sums
+        from enterprise_inference_amd.ops.gemm import columns
+        off = 8
+        wide = torch.randn(3, 6, off + F + 5 + (-(off + F + 5)) % 4, generator=g)
+        wide[:, :, off:off + F] = part
+        got = activation.xielu(columns(SplitK(wide.to(device), 3, 6, wide.shape[2]), off, F),
+                               pq.to(device))
+        assert np.allclose(_np(got), want, atol=loose, rtol=loose), (F, p, q, "partial columns")
 
 
 def case_sigmoid_gate(device, dtype):
