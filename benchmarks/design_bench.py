@@ -122,7 +122,7 @@ def gapidra_config(z: dict) -> dict:
            "mixer": {"heads": H, "kv_heads": G, "dim": D, "vdim": D, "scale": D ** -0.5,
                      "mask": {"size": z["window"]},
                      "rot": {"base": 1e6, "dims": D // 2,
-                             "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0,
+                             "scaling": {"factor": 4.0, "original": 8192, "fast": 32.0,
                                          "slow": 1.0}}}}
     lat = {"type": "latent_attention", "mlp": mlp,
            "mixer": {"heads": H, "dim": D - z["rot"], "rot_dim": z["rot"], "vdim": D,

@@ -155,7 +155,7 @@ def case_qk_rope_cache(device, dtype):
     g = torch.Generator().manual_seed(4)
     for mq, mk, D, vw, rdims, half, scaling, split in (
             (4, 2, 16, 24, 8, False, C.YARN, 0), (6, 2, 10, 14, 10, True, None, 0),
-            (2, 2, 96, 40, 24, False, None, 0), (1, 1, 6, 5, 0, False, None, 0),
+            (2, 2, 80, 40, 20, False, None, 0), (1, 1, 6, 5, 0, False, None, 0),
             (4, 2, 16, 24, 16, False, C.YARN, 3), (3, 1, 24, 20, 6, True, C.YARN, 2)):
         T, bs, nb = 7, 4, 5
         k_off, v_off = 3, 3 + mk * D
