@@ -72,7 +72,8 @@ class GapidraLayer(nn.Module):
         elif self.kind == "attention":
             self.mix = SigmoidWindowAttentionMixer(
                 width, m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m.get("vdim", m["dim"]),
-                m["scale"], window, int(rot.get("dims", 0)), float(rot.get("base", 10000.0)),
+                m["scale"], window, int(rot.get("dims", m["dim"] if rot else 0)),
+                float(rot.get("base", 10000.0)),
                 rot.get("scaling"), eps, dtype, device, extra_rows=ff)
         else:
             raise ValueError(f"unknown Gapidra layer type {self.kind!r}")
