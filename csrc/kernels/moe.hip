@@ -526,30 +526,39 @@ EIA_API int eia_moe_combine_sk(const float* part, int sk, int rows, const float*
 }
 
 // ---------------------------------------------------------------------------------------------
-// Group-limited sigmoid routing: logits z = W_r x in fp32, scores s = sigmoid(z); the experts
-// form `ngroups` equal groups of neighbours, a group scores the sum of its two largest s, only
-// experts of the `keep` best groups are eligible, the `k` largest eligible scores win and weigh
-// s * route_scale (not renormalised).  Ties go to the lower index.  One wave per token: lanes
-// split the width for the dot products; up to 64 experts the lanes then rank themselves with
-// shuffles (lane e = expert e), above that lane 0 selects serially (E <= 256).
+// Group-limited routing: logits z = W_r x in fp32; scores s = sigmoid(z) (scoring 0) or
+// softmax(z) over all E outputs (scoring 1).  Selection ranks the choice scores c = s + corr
+// (corr: an fp32 correction per output, nullable), the weights are the plain scores.  The outputs
+// form `ngroups` equal groups of neighbours; a group scores the sum of its two largest c (gmode 0)
+// or its largest c (gmode 1); only outputs of the `keep` best groups are eligible, the `k` largest
+// eligible c win and weigh s * route_scale (not renormalised).  Choice scores may be negative.
+// Ties go to the lower index.  Outputs n_real .. E-1 are identity experts (no weights: the
+// consumer adds the token's input times their weight): their ids are reported like the others
+// and the sum of their chosen weights lands in ident_w[t] (nullable).  wsg (nullable): one more
+// row [H]; sgate[t] = sigmoid(wsg . x), a token's gate for an always-on expert.
+// One wave per token: lanes split the width for the dot products; up to 64 outputs the lanes then
+// rank themselves with shuffles (lane e = output e), above that lane 0 selects serially (E <= 256).
 template <typename T>
 __global__ void __launch_bounds__(256)
 route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr, int H, int T_,
                      int E, int k, int ngroups, int keep, float route_scale,
                      float* __restrict__ tw, int* __restrict__ ids,
-                     const int* __restrict__ row_len, int extra) {
+                     const int* __restrict__ row_len, int extra, int scoring, int gmode,
+                     const float* __restrict__ corr, int n_real, float* __restrict__ ident_w,
+                     const T* __restrict__ wsg, float* __restrict__ sgate) {
   // extra = 1: one more output column per token naming expert E with weight 1 (an always-on
   // expert stored behind the routed ones); "nowhere" is then E + 1
   const int ko = k + extra, none = E + extra;
   __shared__ float sc[4][256];
+  __shared__ float ch[4][256];
   __shared__ unsigned char ok[4][256];
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + wave;
   if (t >= T_) return;
   const T* xr = x + (long)t * ldx;
-  float mine = -1.f;                           // lane e keeps expert e's score (E <= 64)
+  float mine = -INFINITY;                      // lane e keeps output e's logit (E <= 64)
   const bool vec8 = (H & 7) == 0 && (ldx & 7) == 0;
-  for (int e0 = 0; e0 < E; e0 += 8) {          // eight experts per pass over the token's row
+  for (int e0 = 0; e0 < E; e0 += 8) {          // eight outputs per pass over the token's row
     float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if constexpr (sizeof(T) == 2) {
       if (vec8) {                              // 16-byte loads: 8 consecutive channels per lane
@@ -578,24 +587,38 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
     for (int j = 0; j < 8; ++j) {
       const float v = wave_sum(p[j]);             // every lane holds the total
       if (e0 + j < E) {
-        const float sg = 1.0f / (1.0f + expf(-v));
-        if (lane == 0) sc[wave][e0 + j] = sg;
-        if (lane == e0 + j) mine = sg;
+        if (lane == 0) sc[wave][e0 + j] = v;
+        if (lane == e0 + j) mine = v;
       }
     }
   }
+  if (wsg) {
+    float p = 0.f;
+    for (int c = lane; c < H; c += 64) p += ld_f32<T>(xr, c) * ld_f32<T>(wsg, c);
+    p = wave_sum(p);
+    if (lane == 0) sgate[t] = 1.0f / (1.0f + expf(-p));
+  }
+  const bool pad = row_len && row_len[t] == 0;
+  const int per = E / ngroups;
+  const int gtop = gmode == 1 ? 1 : 2;
   if (E <= 64) {
-    // lane e = expert e: ranks by counting better lanes (ties to the lower index), no LDS
-    const bool pad = row_len && row_len[t] == 0;
-    const int per = E / ngroups;
+    // lane e = output e: ranks by counting better lanes (ties to the lower index), no LDS
     const bool real = lane < E;
+    if (scoring == 1) {
+      const float mx = wave_max(mine);            // (lanes >= E hold -inf)
+      const float ex = real ? expf(mine - mx) : 0.f;
+      mine = ex / wave_sum(ex);
+    } else {
+      mine = real ? 1.0f / (1.0f + expf(-mine)) : 0.f;
+    }
+    const float cme = real ? mine + (corr ? corr[lane] : 0.f) : -INFINITY;
     const int grp = real ? lane / per : -1;
     int r = 0;
     for (int o = 0; o < E; ++o) {
-      const float so = __shfl(mine, o, 64);
-      if (real && o / per == grp && (so > mine || (so == mine && o < lane))) ++r;
+      const float so = __shfl(cme, o, 64);
+      if (real && o / per == grp && (so > cme || (so == cme && o < lane))) ++r;
     }
-    const float contrib = (real && r < 2) ? mine : 0.f;
+    const float contrib = (real && r < gtop) ? cme : 0.f;
     float gsum = 0.f;
     for (int o = 0; o < E; ++o) {
       const float co = __shfl(contrib, o, 64);
@@ -609,17 +632,18 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
     const bool elig = real && grank < keep;
     int fr = 0;
     for (int o = 0; o < E; ++o) {
-      const float so = __shfl(mine, o, 64);
+      const float so = __shfl(cme, o, 64);
       const int eo = __shfl((int)elig, o, 64);
-      if (eo && (so > mine || (so == mine && o < lane))) ++fr;
+      if (eo && (so > cme || (so == cme && o < lane))) ++fr;
     }
+    const bool won = !pad && elig && fr < k;
     if (pad) {
       if (lane < ko) {
         ids[(long)t * ko + lane] = none;
         tw[(long)t * ko + lane] = 0.f;
       }
     } else {
-      if (elig && fr < k) {
+      if (won) {
         ids[(long)t * ko + fr] = lane;
         tw[(long)t * ko + fr] = mine * route_scale;
       }
@@ -628,69 +652,87 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
         tw[(long)t * ko + k] = 1.f;
       }
     }
+    if (ident_w) {
+      const float iw = wave_sum((won && lane >= n_real) ? mine * route_scale : 0.f);
+      if (lane == 0) ident_w[t] = iw;
+    }
     return;
   }
   if (lane != 0) return;
   float* s = sc[wave];
+  float* c = ch[wave];
   unsigned char* el = ok[wave];
-  const bool pad = row_len && row_len[t] == 0;
-  const int per = E / ngroups;
+  if (scoring == 1) {
+    float mx = -INFINITY, sum = 0.f;
+    for (int e = 0; e < E; ++e) mx = fmaxf(mx, s[e]);
+    for (int e = 0; e < E; ++e) { s[e] = expf(s[e] - mx); sum += s[e]; }
+    for (int e = 0; e < E; ++e) s[e] /= sum;
+  } else {
+    for (int e = 0; e < E; ++e) s[e] = 1.0f / (1.0f + expf(-s[e]));
+  }
+  for (int e = 0; e < E; ++e) c[e] = s[e] + (corr ? corr[e] : 0.f);
   // group scores in place of a separate array: pick `keep` groups one by one
   for (int e = 0; e < E; ++e) el[e] = 0;
   for (int r = 0; r < keep; ++r) {
     int best = -1;
     float bv = 0.f;
     for (int g = 0; g < ngroups; ++g) {
-      if (el[g * per]) continue;            // group already taken (its first expert is marked)
+      if (el[g * per]) continue;            // group already taken (its first output is marked)
       float m1 = -INFINITY, m2 = -INFINITY;
       for (int e = g * per; e < (g + 1) * per; ++e) {
-        const float v = s[e];
+        const float v = c[e];
         if (v > m1) { m2 = m1; m1 = v; } else if (v > m2) m2 = v;
       }
-      const float gs = m1 + (per > 1 ? m2 : 0.f);
+      const float gs = m1 + ((per > 1 && gtop == 2) ? m2 : 0.f);
       if (best < 0 || gs > bv) { best = g; bv = gs; }
     }
     if (best < 0) break;
     for (int e = best * per; e < (best + 1) * per; ++e) el[e] = 1;
   }
+  float iw = 0.f;
   for (int r = 0; r < k; ++r) {
     int best = -1;
     float bv = 0.f;
     for (int e = 0; e < E; ++e)
-      if (el[e] == 1 && (best < 0 || s[e] > bv)) { best = e; bv = s[e]; }
+      if (el[e] == 1 && (best < 0 || c[e] > bv)) { best = e; bv = c[e]; }
     if (best < 0 || pad) {
       ids[(long)t * ko + r] = none;         // routes nowhere
       tw[(long)t * ko + r] = 0.f;
     } else {
       el[best] = 2;
       ids[(long)t * ko + r] = best;
-      tw[(long)t * ko + r] = bv * route_scale;
+      tw[(long)t * ko + r] = s[best] * route_scale;
+      if (best >= n_real) iw += s[best] * route_scale;
     }
   }
+  if (ident_w) ident_w[t] = iw;
   if (extra) {
     ids[(long)t * ko + k] = pad ? none : E;
     tw[(long)t * ko + k] = pad ? 0.f : 1.f;
   }
 }
 
-// x [T, H] (row stride ldx) and wr [E, H] in bf16 (is_bf16) or fp32 -> tw fp32 [T, k], ids [T, k].
+// x [T, H] (row stride ldx), wr [E, H] and wsg [H] in bf16 (is_bf16) or fp32 -> tw fp32 [T, k],
+// ids [T, k], ident_w fp32 [T], sgate fp32 [T].
 EIA_API int eia_moe_route_grouped(const void* x, long ldx, const void* wr, int H, int T, int E,
                                   int k, int ngroups, int keep, float route_scale, float* tw,
                                   int* ids, const int* row_len, int extra, int is_bf16,
-                                  hipStream_t st) {
+                                  int scoring, int gmode, const float* corr, int n_real,
+                                  float* ident_w, const void* wsg, float* sgate, hipStream_t st) {
   if (E < 1 || E > 256 || k < 1 || ngroups < 1 || E % ngroups || keep < 1 || keep > ngroups ||
-      k > keep * (E / ngroups) || (extra != 0 && extra != 1))
+      k > keep * (E / ngroups) || (extra != 0 && extra != 1) || (scoring != 0 && scoring != 1) ||
+      (gmode != 0 && gmode != 1) || n_real < 0 || n_real > E || (wsg && !sgate))
     return EIA_BAD_SHAPE;
   if (T <= 0) return EIA_OK;
   dim3 grid((T + 3) / 4), block(256);
   if (is_bf16)
     hipLaunchKernelGGL((route_grouped_kernel<bf16_t>), grid, block, 0, st, (const bf16_t*)x, ldx,
                        (const bf16_t*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,
-                       extra);
+                       extra, scoring, gmode, corr, n_real, ident_w, (const bf16_t*)wsg, sgate);
   else
     hipLaunchKernelGGL((route_grouped_kernel<float>), grid, block, 0, st, (const float*)x, ldx,
                        (const float*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,
-                       extra);
+                       extra, scoring, gmode, corr, n_real, ident_w, (const float*)wsg, sgate);
   EIA_LAUNCH_CHECK();
 }
 

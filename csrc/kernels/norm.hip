@@ -494,3 +494,102 @@ EIA_API int eia_add_rms(const void* y1, long ld1, const float* p1, int sk1, cons
 #undef ADD_RMS_LAUNCH
   EIA_LAUNCH_CHECK();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Boundary of a sublayer whose residual is kept as NS streams joined by hyper-connections, one
+// launch and one workgroup per token row.  X fp32 [rows, NS, W], updated in place:
+//
+//   X_j <- sum_s mix[s, j] X_s + ymult * outw[j] * y            (y given; all streams at once)
+//   u    = sum_j in_next[j] X_j;   h = u / sqrt(mean(u^2) + eps) * (w_off + w_next)   (h given)
+//
+// y is a stored row (type T) or the fp32 split-K partials [sk, rows, W] (+ bias) of the GEMM that
+// produced it, summed here.  mix [NS, NS] (from, to), outw [NS] and in_next [NS] are fp32 device
+// arrays.  NS = 1 with mix = outw = in_next = 1 is the plain residual sum.  All arithmetic fp32.
+constexpr int HC_MAX = 8;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+hyper_step_kernel(float* __restrict__ X, int NS, int W, const T* __restrict__ y, long ldy,
+                  const float* __restrict__ part, int sk, long pstride,
+                  const T* __restrict__ ybias, const float* __restrict__ mix,
+                  const float* __restrict__ outw, float ymult, const float* __restrict__ in_next,
+                  const T* __restrict__ w_next, float w_off, T* __restrict__ h, long ldh,
+                  float eps) {
+  __shared__ float scratch[4];
+  extern __shared__ float u_s[];                    // [W] when h is given
+  const long row = blockIdx.x;
+  float* xr = X + row * (long)NS * W;
+  const bool upd = y || part;
+  float mx[HC_MAX][HC_MAX], ow[HC_MAX], iw[HC_MAX];
+#pragma unroll
+  for (int s = 0; s < HC_MAX; ++s) {
+    ow[s] = (upd && s < NS) ? ymult * outw[s] : 0.f;
+    iw[s] = (h && s < NS) ? in_next[s] : 0.f;
+#pragma unroll
+    for (int j = 0; j < HC_MAX; ++j) mx[s][j] = (upd && s < NS && j < NS) ? mix[s * NS + j] : 0.f;
+  }
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float xs[HC_MAX];
+#pragma unroll
+    for (int s = 0; s < HC_MAX; ++s) xs[s] = s < NS ? xr[(long)s * W + c] : 0.f;
+    if (upd) {
+      float yv;
+      if (y) {
+        yv = ld_f32<T>(y + row * ldy, c);
+      } else {
+        yv = ybias ? ld_f32<T>(ybias, c) : 0.f;
+        const float* p = part + row * (long)W + c;
+        for (int z = 0; z < sk; ++z) yv += p[z * pstride];
+      }
+      float nx[HC_MAX];
+#pragma unroll
+      for (int j = 0; j < HC_MAX; ++j) {
+        float v = ow[j] * yv;
+#pragma unroll
+        for (int s = 0; s < HC_MAX; ++s) v += mx[s][j] * xs[s];
+        nx[j] = v;
+      }
+#pragma unroll
+      for (int j = 0; j < HC_MAX; ++j) {
+        if (j < NS) xr[(long)j * W + c] = nx[j];
+        xs[j] = nx[j];
+      }
+    }
+    if (h) {
+      float u = 0.f;
+#pragma unroll
+      for (int j = 0; j < HC_MAX; ++j) u += iw[j] * xs[j];
+      u_s[c] = u;
+      ss += u * u;
+    }
+  }
+  if (!h) return;
+  const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)W + eps);
+  for (int c = threadIdx.x; c < W; c += blockDim.x)
+    st_f32<T>(h + row * ldh, c, u_s[c] * inv * (w_off + ld_f32<T>(w_next, c)));
+}
+
+// X fp32 [rows, NS, W] contiguous; y, ybias, w_next and h are bf16 when is_bf16 else fp32.
+EIA_API int eia_hyper_step(float* X, int NS, int W, const void* y, long ldy, const float* part,
+                           int sk, const void* ybias, const float* mix, const float* outw,
+                           float ymult, const float* in_next, const void* w_next, float w_off,
+                           void* h, long ldh, float eps, int rows, int is_bf16, hipStream_t st) {
+  if (rows < 0 || W < 1 || NS < 1 || NS > HC_MAX || !X || (y && part) || (part && sk < 1) ||
+      ((y || part) && (!mix || !outw)) || (h && (!w_next || !in_next)))
+    return EIA_BAD_SHAPE;
+  if ((size_t)W * sizeof(float) > 64 * 1024) return EIA_UNSUPPORTED;
+  if (rows == 0) return EIA_OK;
+  const int threads = W >= 1024 ? 256 : (W >= 512 ? 128 : 64);
+  const size_t lds = h ? sizeof(float) * W : 0;
+  const long ps = (long)rows * W;
+  if (is_bf16)
+    hipLaunchKernelGGL((hyper_step_kernel<bf16_t>), dim3(rows), dim3(threads), lds, st, X, NS, W,
+                       (const bf16_t*)y, ldy, part, sk, ps, (const bf16_t*)ybias, mix, outw, ymult,
+                       in_next, (const bf16_t*)w_next, w_off, (bf16_t*)h, ldh, eps);
+  else
+    hipLaunchKernelGGL((hyper_step_kernel<float>), dim3(rows), dim3(threads), lds, st, X, NS, W,
+                       (const float*)y, ldy, part, sk, ps, (const float*)ybias, mix, outw, ymult,
+                       in_next, (const float*)w_next, w_off, (float*)h, ldh, eps);
+  EIA_LAUNCH_CHECK();
+}

@@ -13,8 +13,11 @@
 //   p      = softmax over the visible keys, per map;  a_m = sum_j p_mj v_j
 //   wmode 1: p = sigmoid(s_m + bias[m]) for every visible key, not normalised over the keys
 //            (bias == nullptr: 0; no head mixing, P == 1)
+//   sink (wmode 0, nullable): exp(sink[m]) joins map m's softmax denominator -- a term without a
+//            key or a value, not scaled, counted once.  The running (max, sum) of a row simply
+//            starts at (sink, 1) instead of (-inf, 0); with key partitions, in partition 0.
 //
-// Epilogue 0: out[h] = a_h * sigmoid(gate[h])   (gate == nullptr: out = a; P must be 1)
+// Epilogue 0: out[h] = a_h * sigmoid(gate[h]) * post   (gate == nullptr: no gate; P must be 1)
 // Epilogue 1: o = a_{2h} - lam * a_{2h+1};  out[h] = o / sqrt(mean(o^2) + eps) * post   (P == 2;
 //             lam is read from device memory, so a captured launch follows a weight reload)
 //
@@ -253,6 +256,7 @@ struct WinAttnArgs {
   float* part_acc; float* part_ml;  // [rows, M, nparts, Dv] and [rows, M, nparts, 2] partials
   int wmode;                        // 0: softmax; 1: sigmoid(score + bias), un-normalised
   const float* bias;                // [M] or null (wmode 1)
+  const float* sink;                // [M] or null (wmode 0)
 };
 
 // The visible keys of a 16-query tile as absolute 32-key blocks: the blocks of the kept first
@@ -327,7 +331,10 @@ window_attn_kernel(const WinAttnArgs a) {
     const int nkeys = nsink + pos - lo + 1;
     __syncthreads();                                   // previous query's LDS reads are over
     for (int c = tid; c < M * D; c += 256) qs[c] = ld_f32<T>(q + row * a.ldq, c);
-    for (int m = tid; m < M; m += 256) { mrun[m] = -INFINITY; lrun[m] = 0.f; }
+    for (int m = tid; m < M; m += 256) {
+      mrun[m] = a.sink ? a.sink[m] : -INFINITY;
+      lrun[m] = a.sink ? 1.f : 0.f;
+    }
     float acc[WA_ACC];
 #pragma unroll
     for (int i = 0; i < WA_ACC; ++i) acc[i] = 0.f;
@@ -401,7 +408,7 @@ window_attn_kernel(const WinAttnArgs a) {
       for (int i = 0; i < WA_ACC; ++i) {
         const int idx = tid + i * 256;
         if (idx < M * Dv) {
-          float v = acc[i] / lrun[idx / Dv];
+          float v = acc[i] / lrun[idx / Dv] * a.post;
           if (gate) v *= 1.0f / (1.0f + expf(-ld_f32<T>(gate + row * a.ldg, idx)));
           st_f32<T>(out + row * a.ldo, idx, v);
         }
@@ -442,21 +449,22 @@ EIA_API int eia_window_attn(const void* q, long ldq, const void* kc, const void*
                             const float* talk, const void* gate, long ldg, void* out, long ldo,
                             int H, int G, int P, int D, int Dv, int bs, int window, int keep,
                             int qb, int epilogue, const float* lam, float eps, float post,
-                            int wmode, const float* bias, int is_bf16, hipStream_t st) {
+                            int wmode, const float* bias, const float* sink, int is_bf16,
+                            hipStream_t st) {
   if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || D < 1 || Dv < 1 || bs < 1 ||
       keep < 0 || qb < 1 || !q || !kc || !vc || !bt || !positions || !mult || !out)
     return EIA_BAD_SHAPE;
   if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
   if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam)))
     return EIA_BAD_SHAPE;
-  if ((wmode != 0 && wmode != 1) || (wmode == 1 && (talk || P != 1))) return EIA_BAD_SHAPE;
+  if ((wmode != 0 && wmode != 1) || (wmode == 1 && (talk || P != 1 || sink))) return EIA_BAD_SHAPE;
   const int M = H * P;
   const size_t lds = wa_lds_bytes(M, D, Dv);
   if (M * Dv > 256 * WA_ACC || lds > 64 * 1024) return EIA_UNSUPPORTED;
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
                 out, ldo, H, G, P, D, Dv, bs, window, keep, qb, epilogue, lam, eps, post, 1, 2,
-                nullptr, nullptr, wmode, bias};
+                nullptr, nullptr, wmode, bias, sink};
   if (is_bf16)
     hipLaunchKernelGGL((window_attn_kernel<bf16_t>), dim3(n_items), dim3(256), lds, st, a);
   else
@@ -556,8 +564,9 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
   float mrun[MW], lrun[MW];
 #pragma unroll
   for (int m = 0; m < MW; ++m) {
-    mrun[m] = -1e30f;
-    lrun[m] = 0.f;
+    const bool snk = !SIG && a.sink && blockIdx.z == 0;
+    mrun[m] = snk ? a.sink[hs * P + m] : -1e30f;
+    lrun[m] = snk ? 1.f : 0.f;
 #pragma unroll
     for (int t = 0; t < NDV; ++t) acc[m][t] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
@@ -797,7 +806,7 @@ window_attn_mfma_kernel(const WinAttnArgs a) {
     const bf16_t* gate = (const bf16_t*)a.gate;
 #pragma unroll
     for (int m = 0; m < MW; ++m) {
-      const float inv = 1.0f / lrun[m];
+      const float inv = a.post / lrun[m];
 #pragma unroll
       for (int t = 0; t < NDV; ++t) {
         if (t < ndv) {
@@ -877,8 +886,8 @@ window_attn_merge_kernel(const WinAttnArgs a) {
   float r0, r1;
   if (a.epilogue == 0) {
     const bf16_t* gate = (const bf16_t*)a.gate;
-    r0 = o[0][0];
-    r1 = o[0][1];
+    r0 = o[0][0] * a.post;
+    r1 = o[0][1] * a.post;
     if (gate) {
       if (lane < Dv) r0 *= 1.0f / (1.0f + __expf(-bf2f(gate[row * a.ldg + h * Dv + lane])));
       if (lane + 64 < Dv) r1 *= 1.0f / (1.0f + __expf(-bf2f(gate[row * a.ldg + h * Dv + lane + 64])));
@@ -919,13 +928,14 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
                                  void* out, long ldo, int H, int G, int P, int D, int Dv, int bs,
                                  int window, int keep, int epilogue, const float* lam, float eps,
                                  float post, int wmode, const float* bias, int nparts,
-                                 float* part_acc, float* part_ml, hipStream_t st) {
+                                 float* part_acc, float* part_ml, const float* sink,
+                                 hipStream_t st) {
   if (n_items < 0 || H < 1 || G < 1 || H % G || (P != 1 && P != 2) || bs < 1 || keep < 0 || !q ||
       !kc || !vc || !bt || !positions || !mult || !out)
     return EIA_BAD_SHAPE;
   if ((cu == nullptr) != (work == nullptr)) return EIA_BAD_SHAPE;
   if ((epilogue == 1) != (P == 2) || (epilogue == 1 && (gate || !lam))) return EIA_BAD_SHAPE;
-  if ((wmode != 0 && wmode != 1) || (wmode == 1 && (talk || P != 1))) return EIA_BAD_SHAPE;
+  if ((wmode != 0 && wmode != 1) || (wmode == 1 && (talk || P != 1 || sink))) return EIA_BAD_SHAPE;
   if (!eia_window_attn_mfma_ok(H, G, P, D, Dv, bs, talk != nullptr)) return EIA_UNSUPPORTED;
   if (ldq % 8 || ldo % 4) return EIA_BAD_SHAPE;
   // key partitions: decode rows only (a row is its own work item), partials in the workspace
@@ -934,7 +944,7 @@ EIA_API int eia_window_attn_mfma(const void* q, long ldq, const void* kc, const 
   if (n_items == 0) return EIA_OK;
   WinAttnArgs a{q, ldq, kc, vc, bt, ldbt, positions, cu, work, lens, mult, slope, talk, gate, ldg,
                 out, ldo, H, G, P, D, Dv, bs, window, keep, 16, epilogue, lam, eps, post, nparts,
-                2, part_acc, part_ml, wmode, bias};
+                2, part_acc, part_ml, wmode, bias, sink};
   // raw-score buffers of the head-mixing form: two (one barrier per block) while they fit 48 KiB
   if (talk) a.raw_bufs = (size_t)2 * H * P * 128 * sizeof(f32x4) > 48 * 1024 ? 1 : 2;
   // sigmoid weights: a wave takes two heads of one kv head where the grouping allows it, so the

@@ -74,7 +74,11 @@ _SIGNATURES = {
     "eia_token_shift_mix": [P, P, I, P, IP, IP, I, IP, P, L, I, I, I, S],
     "eia_wkv_scan": [P, P, P, P, L, P, L, P, P, P, P, P, P, I, IP, IP, IP, IP, P, L, F, I, I, I,
                      I, S],
-    "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, I, S],
+    "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, I, I, I, P, I, P, P, P, S],
+    "eia_linear_scan": [P, L, I, I, I, I, I, I, P, P, I, I, F, F, F, F, P, P, P, P, IP, IP, IP, IP,
+                        P, L, F, I, I, I, I, I, I, I, S],
+    "eia_hyper_step": [P, I, I, P, L, P, I, P, P, P, F, P, P, F, P, L, F, I, I, S],
+    "eia_bigram_embed": [IP, P, F, P, I, L, L, IP, IP, IP, I, IP, P, I, I, I, I, I, S],
     "eia_relu2": [P, P, L, I, S],
     "eia_moe_combine_postnorm": [P, L, P, P, I, P, L, P, F, P, P, L, I, I, I, S],
     "eia_gnorm": [P, L, P, I, P, P, P, P, P, P, L, F, I, I, I, I, S],
@@ -82,9 +86,9 @@ _SIGNATURES = {
     "eia_qk_norm_cache": [P, L, P, I, P, I, I, I, I, I, I, I, I, I, P, P, P, L, P, P, P, L, IP, I, F,
                           I, I, S],
     "eia_window_attn": [P, L, P, P, IP, I, IP, IP, IP, IP, I, P, P, P, P, L, P, L, I, I, I, I, I,
-                        I, I, I, I, I, P, F, F, I, P, I, S],
+                        I, I, I, I, I, P, F, F, I, P, P, I, S],
     "eia_window_attn_mfma": [P, L, P, P, IP, I, IP, IP, IP, IP, I, P, P, P, P, L, P, L, I, I, I, I,
-                             I, I, I, I, I, P, F, F, I, P, I, P, P, S],
+                             I, I, I, I, I, P, F, F, I, P, I, P, P, P, S],
     "eia_qk_rope_cache": [P, L, P, I, P, I, I, I, I, I, I, I, P, P, P, I, I, F, IP, P, L, P, P, IP,
                           I, F, I, I, S],
     "eia_add_rms": [P, L, P, I, P, P, L, P, I, P, P, P, P, L, F, I, I, I, S],

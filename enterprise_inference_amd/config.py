@@ -139,10 +139,12 @@ class ModelConfig:
     def from_layer_list(cls, d: Dict[str, Any], name: str = "",
                         tensor_shapes: Optional[Dict[str, Any]] = None) -> "ModelConfig":
         """Designs whose config.json names the architecture in one string and lists the layers
-        one by one (Sekolorn, Vedadra, Gapidra): keys ``architecture``, ``vocab``, ``width``,
-        ``norm.eps`` and ``layers`` (kept whole in ``extra["layers"]``); ``norm``, ``embedding``
-        ({scale}) and an optional ``loop`` ({start, stop, times}: a run of layers repeated with
-        the same weights) are kept whole too.  Sizes the file leaves to the checkpoint (the rank
+        one by one (Sekolorn, Vedadra, Gapidra, Daburax): keys ``architecture``, ``vocab``,
+        ``width``, ``norm.eps`` and ``layers`` (kept whole in ``extra["layers"]``); ``norm``,
+        ``embedding`` ({scale, bigram}) and an optional ``loop`` ({start, stop, times}: a run of
+        layers repeated with the same weights) are kept whole too, as are ``residual_mult`` (a
+        factor on every sublayer output) and ``streams`` (residual copies joined by
+        hyper-connections).  Sizes the file leaves to the checkpoint (the rank
         of a wkv layer's decay branch) come from ``tensor_shapes`` when given."""
         import copy
         layers = copy.deepcopy(d["layers"])
@@ -151,17 +153,20 @@ class ModelConfig:
             if L.get("type") == "wkv" and "decay_rank" not in m:
                 shp = (tensor_shapes or {}).get(f"l{i}.mix.w1")
                 m["decay_rank"] = int(shp[0]) if shp else 64
-        heads = [L["mixer"].get("heads", 1) for L in layers]
+        heads = [(L["mixer"].get("left") or L["mixer"]).get("heads", 1) for L in layers]
         eps = float((d.get("norm") or {}).get("eps", 1e-6))
         return cls(architecture=d["architecture"], hidden_size=int(d["width"]),
                    num_hidden_layers=len(layers), num_attention_heads=max(heads + [1]),
                    vocab_size=int(d["vocab"]), num_key_value_heads=1,
-                   head_dim=max([L["mixer"].get("dim", 1) for L in layers] + [1]),
+                   head_dim=max([(L["mixer"].get("left") or L["mixer"]).get("dim", 1)
+                                 for L in layers] + [1]),
                    max_position_embeddings=1 << 20,      # the design sets no limit
                    rms_norm_eps=eps, layer_norm_eps=eps,
                    name=name, extra={"layers": layers, "norm": dict(d.get("norm") or {}),
                                      "embedding": dict(d.get("embedding") or {}),
-                                     "loop": dict(d["loop"]) if d.get("loop") else None})
+                                     "loop": dict(d["loop"]) if d.get("loop") else None,
+                                     "residual_mult": d.get("residual_mult"),
+                                     "streams": d.get("streams")})
 
     @classmethod
     def from_hf_dict(cls, d: Dict[str, Any], name: str = "") -> "ModelConfig":

@@ -20,6 +20,7 @@ _REGISTRY: Dict[str, str] = {
     "Sekolorn": "sekolorn:SekolornForCausalLM",
     "Vedadra": "vedadra:VedadraForCausalLM",
     "Gapidra": "gapidra:GapidraForCausalLM",
+    "Daburax": "daburax:DaburaxForCausalLM",
     "BertModel": "bert:BertEmbeddingModel",
     "XLMRobertaModel": "bert:BertEmbeddingModel",
     "XLMRobertaForSequenceClassification": "bert:CrossEncoderModel",

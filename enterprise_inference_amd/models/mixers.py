@@ -20,7 +20,18 @@ returns the mixer output in the activation dtype.
 * ``SigmoidWindowAttentionMixer`` -- grouped-query sliding-window attention whose weights are
   ``sigmoid(score + bias_h)``, not normalised over the keys; queries and keys are RMS-normed as
   whole projections and then rotated.
-  All three run on token-major paged K / V rows (``PagedKVRows``, ops/window_attention.py).
+* ``SinkAttentionMixer`` -- grouped-query causal softmax attention with projection biases, a
+  partial rotation with optional position interpolation and a learned per-head sink in the
+  softmax denominator (optionally windowed).
+  All four run on token-major paged K / V rows (``PagedKVRows``, ops/window_attention.py).
+* ``RetentionMixer`` -- linear attention with a fixed decay per head: rotated q / k, a matrix
+  state per head on per-sequence state slots, head RMS norm, SiLU gate.
+* ``MatrixMemoryMixer`` -- a gated matrix memory: exponential input gate and sigmoid forget gate
+  per head with soft-capped pre-activations, stabilised by a running maximum, a normaliser
+  state, head RMS norm with a weight, sigmoid gate.  Both run ops/linear_scan.py.
+* ``ParallelMixer`` -- an attention mixer and a recurrent mixer side by side on the same input:
+  one fused input projection, one output projection over the concatenated heads, the two
+  outputs added with fixed factors.
 """
 
 from __future__ import annotations
@@ -31,6 +42,7 @@ import torch.nn as nn
 from ..ops import activation as act_ops
 from ..ops import gemm
 from ..ops import latent_attention as lat_ops
+from ..ops import linear_scan as scan_ops
 from ..ops import rotary as rot_ops
 from ..ops import window_attention as win_ops
 from ..ops import wkv as wkv_ops
@@ -258,7 +270,7 @@ class _WindowMixerBase(nn.Module):
     maps = 1
 
     def _setup(self, width, heads, kv_heads, dim, vdim, scale, window, keep, eps, parts, bias,
-               dtype, device, norm_sizes=None):
+               dtype, device, norm_sizes=None, norms=True, own_out=True):
         if pstate.tp_size() != 1:
             raise NotImplementedError("window attention mixers run on one rank (no head sharding yet)")
         if heads % kv_heads:
@@ -281,9 +293,9 @@ class _WindowMixerBase(nn.Module):
             self.proj_bias.weight_loader = self._load_part
         # norm weights: one per map entry (shared by the maps), or ``norm_sizes`` = (query, key)
         qn, kn = norm_sizes or (dim, dim)
-        self.q_norm = _plain((qn,), dtype, device)
-        self.k_norm = _plain((kn,), dtype, device)
-        self.o = _plain((width, heads * vdim), dtype, device)
+        self.q_norm = _plain((qn,), dtype, device) if norms else None
+        self.k_norm = _plain((kn,), dtype, device) if norms else None
+        self.o = _plain((width, heads * vdim), dtype, device) if own_out else None
         M = heads * self.maps
         # fp32 constants of the attention launch, refreshed IN PLACE after a weight load
         # (captured decode graphs hold their addresses)
@@ -429,3 +441,266 @@ class SigmoidWindowAttentionMixer(_WindowMixerBase):
         if want_extra:
             return y, gemm.columns(fused, *self.offsets["x"])
         return y
+
+
+class FusedProjection(nn.Module):
+    """One input projection shared by several consumers of the same layer input: named parts
+    (rows each) stacked into one weight, zero-padded to a multiple of 64 rows, with an optional
+    bias over the parts that have one.  ``offsets[name] = (first column, columns)`` of the
+    output row."""
+
+    def __init__(self, width: int, parts, dtype, device, bias_parts=()):
+        super().__init__()
+        self.offsets, n = {}, 0
+        for name, rows in parts:
+            n = -(-n // 8) * 8                       # 16-byte aligned column ranges
+            self.offsets[name] = (n, int(rows))
+            n += int(rows)
+        self.weight = _param((_pad64(n), width), dtype, device)
+        self.weight.data.zero_()
+        self.weight.weight_loader = self._load_part
+        self.bias = None
+        self.bias_parts = tuple(bias_parts)
+        if self.bias_parts:
+            self.bias = _param((_pad64(n),), dtype, device)
+            self.bias.data.zero_()
+            self.bias.weight_loader = self._load_part
+
+    def _load_part(self, param, loaded, shard_id=None):
+        off, rows = self.offsets[shard_id]
+        if loaded.shape[0] != rows or param.data[off:off + rows].shape != loaded.shape:
+            raise ValueError(f"fused projection part {shard_id!r}: shape {tuple(loaded.shape)}")
+        param.data[off:off + rows].copy_(loaded)
+
+    def init_random(self, gen) -> None:
+        """N(0, 1/width) rows for every part, small biases; pad rows stay zero."""
+        w = self.weight
+        w.data.zero_()
+        for name, (off, rows) in self.offsets.items():
+            w.data[off:off + rows].copy_(torch.randn((rows, w.shape[1]), generator=gen,
+                                                     device=w.device, dtype=torch.float32)
+                                         * w.shape[1] ** -0.5)
+            if name in self.bias_parts:
+                self.bias.data[off:off + rows].copy_(
+                    torch.randn((rows,), generator=gen, device=w.device, dtype=torch.float32) * 0.1)
+
+    def forward(self, xb: torch.Tensor, defer_reduce: bool = False):
+        return gemm.linear(xb, self.weight, self.bias, defer_reduce=defer_reduce)
+
+
+class SinkAttentionMixer(_WindowMixerBase):
+    """Grouped-query causal softmax attention: q, k and v carry biases; the first ``rot_dims``
+    entries of every query / key head turn by the position (pairs (2i, 2i+1), or (i, i +
+    rot_dims/2) with ``rot_half``; ``rot_scaling`` as in ops/rotary.py rotary_frequencies, a
+    lone ``factor`` divides every frequency); score = (q . k) * scale; the softmax denominator
+    of head h also holds exp(sink_h), a learned term without key or value; ``window`` 0 sees
+    every earlier token.  The concatenated heads are multiplied by ``out_scale``.
+    ``proj`` / ``prefix``: the q, k, v parts live in a caller's FusedProjection under
+    ``prefix + "q"`` ...; the caller then also owns the output projection, and ``attend`` writes
+    the heads into the caller's buffer."""
+
+    PARTS = ("q", "k", "v")
+
+    @staticmethod
+    def parts(heads, kv_heads, dim, vdim):
+        return [("q", heads * dim), ("k", kv_heads * dim), ("v", kv_heads * vdim)]
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float,
+                 rot_dims: int, rot_base: float, rot_scaling, eps: float, dtype, device,
+                 window: int = 0, rot_half: bool = False, out_scale: float = 1.0,
+                 proj: "FusedProjection" = None, prefix: str = ""):
+        super().__init__()
+        if rot_dims > dim or rot_dims % 2:
+            raise ValueError("rot.dims must be even and at most dim")
+        own = proj is None
+        self._setup(width, heads, kv_heads, dim, vdim, scale, window, 0, eps,
+                    self.parts(heads, kv_heads, dim, vdim) if own else [], own, dtype, device,
+                    norms=False, own_out=own)
+        if not own:
+            self.proj = self.proj_bias = None
+            self.offsets = {n: proj.offsets[prefix + n] for n in self.PARTS}
+        self.rot_dims, self.rot_half = int(rot_dims), rot_half
+        self.inv_freq, self.rot_amp = rot_ops.rotary_frequencies(rot_dims, rot_base, rot_scaling,
+                                                                 device)
+        self.sink = _plain((heads,), dtype, device)
+        self.spec.sink = torch.zeros(heads, dtype=torch.float32, device=device)
+        self.spec.post = float(out_scale)
+
+    def refresh(self) -> None:
+        self.spec.sink.copy_(self.sink.float())
+
+    def attend(self, fused, md: AttentionMetadata, cache: PagedKVRows, out=None):
+        q = win_ops.qk_rope_cache(fused, self.offsets["q"][0], self.offsets["k"][0],
+                                  self.offsets["v"][0], self.heads, self.kv_heads, self.dim,
+                                  self.kv_heads * self.vdim, None, None, self.inv_freq,
+                                  self.rot_dims, self.rot_half, self.rot_amp, md.positions,
+                                  cache.k, cache.v, md.slot_mapping, self.eps)
+        return win_ops.window_attention(q, cache.k, cache.v, md, self.spec, None, out=out)
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache: PagedKVRows):
+        fused = gemm.linear(xb, self.proj, self.proj_bias, defer_reduce=True)
+        # may return gemm.SplitK: the layer's boundary step reduces it
+        return gemm.linear(self.attend(fused, md, cache), self.o, defer_reduce=True)
+
+
+class _ScanMixerBase(nn.Module):
+    """Shared parts of the mixers over ``ScanState`` slots: the fused input projection (their own
+    or a caller's), the scan launch and the output projection."""
+
+    def _setup(self, width, parts, bias_parts, dtype, device, proj, prefix):
+        if pstate.tp_size() != 1:
+            raise NotImplementedError("recurrent mixers run on one rank (no head sharding yet)")
+        self.width = width
+        self.own = proj is None
+        if self.own:
+            self.proj = FusedProjection(width, parts, dtype, device, bias_parts)
+            self.offsets = dict(self.proj.offsets)
+            self.o = _plain((width, self.spec.heads * self.spec.vdim), dtype, device)
+        else:
+            self.proj = self.o = None
+            self.offsets = {n: proj.offsets[prefix + n] for n, _ in parts}
+
+    def state_bytes(self) -> int:
+        return scan_ops.ScanState.slot_bytes(self.spec)
+
+    def allocate_state(self, num_slots: int, device) -> scan_ops.ScanState:
+        return scan_ops.ScanState.allocate(num_slots, self.spec, device)
+
+    def refresh(self) -> None:
+        pass
+
+    def _scan(self, fused, md, state, norm_w, out):
+        from ..ops.gemm import SplitK
+        if isinstance(fused, SplitK):
+            fused = fused.materialize() if fused.part.is_cuda else \
+                fused.part.sum(0) + (fused.bias.float() if fused.bias is not None else 0.0)
+        o = self.offsets
+        return scan_ops.linear_scan(
+            fused, o["q"][0], o["k"][0], o["v"][0], o["g"][0], self.spec, state, md.seq_slots,
+            md.seq_cu, md.num_seqs, md.positions,
+            md.decode_seq_lens if md.seq_cu is None else None, norm_w,
+            o["i"][0] if "i" in o else 0, o["f"][0] if "f" in o else 0, out)
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, state):
+        # may return gemm.SplitK: the layer's boundary step reduces it
+        return gemm.linear(self.attend(self.proj(xb), md, state), self.o, defer_reduce=True)
+
+
+class RetentionMixer(_ScanMixerBase):
+    """Linear attention with a fixed decay per head and neither softmax nor denominator:
+    q, k [heads, dim] and v [heads, vdim] without biases; the first ``rot_dims`` entries of q and
+    k turn by the position (pairs (i, i + rot_dims/2), or (2i, 2i+1) with ``rot_half`` False); k
+    is then multiplied by dim^(-1/2);  S_t = decay_h S_(t-1) + k_t v_t^T,  o_t = S_t^T q_t;
+    every head's o is divided by its root mean square; the concatenated heads are multiplied by
+    silu(W_g x) and ``out_scale``."""
+
+    @staticmethod
+    def parts(heads, dim, vdim):
+        return [("q", heads * dim), ("k", heads * dim), ("v", heads * vdim), ("g", heads * vdim)]
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, rot_dims: int,
+                 rot_base: float, rot_scaling, eps: float, dtype, device, rot_half: bool = True,
+                 out_scale: float = 1.0, proj: "FusedProjection" = None, prefix: str = ""):
+        super().__init__()
+        if len(decay) != heads:
+            raise ValueError("retention: one decay per head")
+        if rot_dims > dim or rot_dims % 2:
+            raise ValueError("rot.dims must be even and at most dim")
+        inv_freq, _ = rot_ops.rotary_frequencies(rot_dims, rot_base, rot_scaling, device)
+        self.spec = scan_ops.ScanSpec(
+            heads, dim, vdim, "decay",
+            decay=torch.tensor([float(d) for d in decay], dtype=torch.float32, device=device),
+            inv_freq=inv_freq, rot_dims=int(rot_dims), rot_half=rot_half, qscale=1.0,
+            kscale=float(dim) ** -0.5, gate_act="silu", out_scale=float(out_scale), eps=float(eps))
+        self._setup(width, self.parts(heads, dim, vdim), (), dtype, device, proj, prefix)
+
+    def attend(self, fused, md: AttentionMetadata, state, out=None):
+        return self._scan(fused, md, state, None, out)
+
+
+class MatrixMemoryMixer(_ScanMixerBase):
+    """Gated matrix memory: q = W_q x * dim^(-1/2), k [heads, dim], v [heads, vdim]; per head a
+    log input gate i = cap tanh((W_i x + b_i) / cap) and a log forget gate f = logsigmoid(cap
+    tanh((W_f x + b_f) / cap)); with a running maximum m_t = max(f + m_(t-1), i) (from 0):
+    S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T, n_t likewise with k alone,
+    o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6).  Every head's o is divided by its root mean
+    square; the concatenated heads are multiplied by the weight ``norm``, sigmoid(W_g x) and
+    ``out_scale``."""
+
+    @staticmethod
+    def parts(heads, dim, vdim):
+        return [("q", heads * dim), ("k", heads * dim), ("v", heads * vdim), ("g", heads * vdim),
+                ("i", heads), ("f", heads)]
+
+    BIAS_PARTS = ("i", "f")
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, gate_cap: float, eps: float,
+                 dtype, device, out_scale: float = 1.0, proj: "FusedProjection" = None,
+                 prefix: str = ""):
+        super().__init__()
+        self.spec = scan_ops.ScanSpec(heads, dim, vdim, "exp_gates", cap=float(gate_cap),
+                                      qscale=float(dim) ** -0.5, kscale=1.0, gate_act="sigmoid",
+                                      out_scale=float(out_scale), eps=float(eps))
+        self._setup(width, self.parts(heads, dim, vdim), self.BIAS_PARTS, dtype, device, proj,
+                    prefix)
+        self.norm = _plain((heads * vdim,), dtype, device)
+
+    def attend(self, fused, md: AttentionMetadata, state, out=None):
+        return self._scan(fused, md, state, self.norm, out)
+
+
+class ParallelMixer(nn.Module):
+    """Two mixers side by side on the same input, ``left_scale * left(x) + right_scale *
+    right(x)``: ``left`` a SinkAttentionMixer on paged K / V rows, ``right`` a MatrixMemoryMixer on
+    state slots.  Both read ONE fused input projection and write their (scaled) heads into one
+    row, so one output projection over the concatenated heads adds the two in fp32."""
+
+    def __init__(self, width: int, left: dict, right: dict, left_scale: float, right_scale: float,
+                 eps: float, dtype, device):
+        super().__init__()
+        lp = SinkAttentionMixer.parts(left["heads"], left["kv_heads"], left["dim"], left["vdim"])
+        rp = MatrixMemoryMixer.parts(right["heads"], right["dim"], right["vdim"])
+        self.proj = FusedProjection(
+            width, [("left." + n, r) for n, r in lp] + [("right." + n, r) for n, r in rp], dtype,
+            device, tuple("left." + n for n, _ in lp) +
+            tuple("right." + n for n in MatrixMemoryMixer.BIAS_PARTS))
+        rot = left.get("rot") or {}
+        self.left = SinkAttentionMixer(
+            width, left["heads"], left["kv_heads"], left["dim"], left["vdim"], left["scale"],
+            int(rot.get("dims", 0)), float(rot.get("base", 10000.0)), rot.get("scaling"), eps,
+            dtype, device, window=int((left.get("mask") or {}).get("size", 0)),
+            out_scale=left_scale, proj=self.proj, prefix="left.")
+        self.right = MatrixMemoryMixer(width, right["heads"], right["dim"], right["vdim"],
+                                       right["gate_cap"], eps, dtype, device,
+                                       out_scale=right_scale, proj=self.proj, prefix="right.")
+        self.lw = left["heads"] * left["vdim"]
+        self.rw = right["heads"] * right["vdim"]
+        self.lw_pad = -(-self.lw // 8) * 8           # the right heads start 16-byte aligned
+        # output projection over [left heads | pad | right heads]; the checkpoint's two output
+        # matrices load into its column ranges
+        self.o = _param((width, self.lw_pad + self.rw), dtype, device)
+        self.o.data.zero_()
+        self.o.weight_loader = self._load_o
+
+    def _load_o(self, param, loaded, shard_id=None):
+        off, n = (0, self.lw) if shard_id == "left" else (self.lw_pad, self.rw)
+        if loaded.shape != (param.shape[0], n):
+            raise ValueError(f"parallel mixer {shard_id}.o: shape {tuple(loaded.shape)}")
+        param.data[:, off:off + n].copy_(loaded)
+
+    def refresh(self) -> None:
+        self.left.refresh()
+        self.right.refresh()
+
+    def forward(self, xb: torch.Tensor, md: AttentionMetadata, cache):
+        """cache: (PagedKVRows of the left mixer, ScanState of the right one)."""
+        kv, state = cache
+        fused = self.proj(xb)
+        T = xb.shape[0]
+        heads = torch.empty(T, self.lw_pad + self.rw, dtype=xb.dtype, device=xb.device)
+        if self.lw_pad != self.lw:
+            heads[:, self.lw:self.lw_pad].zero_()
+        self.left.attend(fused, md, kv, out=heads[:, :self.lw])
+        self.right.attend(fused, md, state, out=heads[:, self.lw_pad:])
+        # may return gemm.SplitK: the layer's boundary step reduces it
+        return gemm.linear(heads, self.o, defer_reduce=True)

@@ -289,6 +289,77 @@ class GroupRoutedMoE(nn.Module):
         return moe_ops.combine_post_norm(h2, tw, inv, shared, norm_w, eps, resid)
 
 
+class GroupLimitedMoE(nn.Module):
+    """Gated experts  W_down (act(W_gate x) * (W_up x))  behind a group-limited router
+    (ops/moe.py route_grouped + fused_moe): fp32 router logits over ``num_experts + identity``
+    outputs, softmax (or sigmoid) scores, a stored per-output ``correction`` that is added for
+    the selection only, groups of neighbouring outputs of which the best ``keep_groups`` (by
+    their largest, or two largest, corrected scores) stay eligible, ``top_k`` winners weighing
+    their plain scores times ``route_scale`` without renormalisation.  The last ``identity``
+    outputs are identity experts: no weights, their output is the input.  An optional shared
+    expert of size ``shared_inter`` runs for every token, times sigmoid(w_sg . x) when
+    ``shared_gate``.  One rank."""
+
+    def __init__(self, hidden: int, inter: int, num_experts: int, top_k: int, num_groups: int = 1,
+                 keep_groups: int = 1, identity: int = 0, shared_inter: int = 0,
+                 shared_gate: bool = True, scoring: str = "softmax", group_score: str = "max",
+                 route_scale: float = 1.0, act: str = "silu", dtype=torch.bfloat16, device=None):
+        super().__init__()
+        if state.tp_size() != 1:
+            raise NotImplementedError("GroupLimitedMoE runs on one rank")
+        n_out = num_experts + identity
+        if n_out % num_groups or not (1 <= keep_groups <= num_groups) or \
+                top_k > keep_groups * (n_out // num_groups):
+            raise ValueError("router groups do not fit the output count / top-k")
+        self.E, self.identity, self.k = num_experts, int(identity), top_k
+        self.groups, self.keep = num_groups, keep_groups
+        self.scoring, self.group_score, self.route_scale = scoring, group_score, float(route_scale)
+        self.act = act
+        self.router = _param((n_out, hidden), dtype, device)
+        self.correction = _param((n_out,), dtype, device)
+        self.correction.data.zero_()
+        self.router.weight_loader = self.correction.weight_loader = \
+            lambda p, t, sid=None: p.data.copy_(t)
+        # fp32 copy of the correction for the router launch, refreshed IN PLACE after a weight
+        # load (captured decode graphs hold its address)
+        self.corr_f32 = torch.zeros(n_out, dtype=torch.float32, device=device)
+        self.w13 = _param((num_experts, 2 * inter, hidden), dtype, device)     # [gate; up] rows
+        self.w2 = _param((num_experts, hidden, inter), dtype, device)
+        self.w13.weight_loader = self._load_w13
+        self.w2.weight_loader = lambda p, t, sid=None: p.data[sid].copy_(t)
+        self.I = inter
+        self.shared = LlamaMLP(hidden, shared_inter, act, dtype, device) if shared_inter else None
+        self.shared_gate = None
+        if self.shared is not None and shared_gate:
+            self.shared_gate = _param((hidden,), dtype, device)
+            self.shared_gate.weight_loader = lambda p, t, sid=None: p.data.copy_(t.reshape(-1))
+
+    def _load_w13(self, param, loaded, shard_id):
+        e, which = shard_id
+        off = 0 if which == "gate" else self.I
+        param.data[e, off:off + self.I].copy_(loaded)
+
+    def refresh(self) -> None:
+        self.corr_f32.copy_(self.correction.float())
+
+    def forward(self, x: torch.Tensor, md=None) -> torch.Tensor:
+        row_len = None
+        if md is not None and md.num_prefill_tokens == 0 and md.decode_seq_lens is not None:
+            row_len = md.decode_seq_lens          # bucket-padding rows route nowhere
+        r = moe_ops.route_grouped(x, self.router, self.k, self.groups, self.keep,
+                                  self.route_scale, row_len, scoring=self.scoring,
+                                  group_score=self.group_score, correction=self.corr_f32,
+                                  identity=self.identity, gate_w=self.shared_gate)
+        tw, ids = r[0], r[1]
+        ident_w, sgate = (r[2], r[3]) if len(r) == 4 else (None, None)
+        routed = moe_ops.fused_moe(x, self.w13, self.w2, tw, ids, (0, self.E), act=self.act)
+        shared = None
+        if self.shared is not None:
+            shared = self.shared(x)
+            shared = shared.materialize() if hasattr(shared, "materialize") else shared
+        return moe_ops.finish_gated(routed, x, ident_w, shared, sgate)
+
+
 class MixtralForCausalLM(LlamaForCausalLM):
     def __init__(self, cfg: ModelConfig, dtype=torch.bfloat16, device=None):
         super().__init__(cfg, dtype, device, layer_factory=lambda i: LlamaDecoderLayer(

@@ -1,0 +1,199 @@
+"""Linear-attention recurrences with one decay number per head and token, on per-sequence state
+slots -> csrc/kernels/linear_scan.hip.
+
+Per head a matrix state S [dk, dv] (fp32, slot-resident) that every token scales and adds an
+outer product to; the token's output reads the updated state:
+
+    S_t = a_t S_(t-1) + b_t k_t v_t^T,        o_t = S_t^T q_t
+
+* ``mode="decay"`` (retention): a_t = decay[h], b_t = 1.
+* ``mode="exp_gates"`` (matrix memory with exponential gating): per head two gate
+  pre-activations x_i, x_f per token; i = cap tanh(x_i / cap), f = logsigmoid(cap tanh(x_f /
+  cap)); a running maximum m_t = max(f + m_(t-1), i) (m starts at 0) keeps the exponentials
+  bounded: a_t = exp(f + m_(t-1) - m_t), b_t = exp(i - m_t); a normaliser n_t = a_t n_(t-1) +
+  b_t k_t divides the output, o_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
+
+q and k may be rotated by the token's position on their first ``rot_dims`` entries and are then
+scaled; every head's output is divided by its root mean square, multiplied by an optional weight,
+by silu or sigmoid of the gate columns and by ``out_scale``.
+
+A sequence whose first row of the step is position 0 starts from the initial state whatever its
+slot held, so freed slots are reused without clearing.  Batch layout: sequence ``s`` owns rows
+``[cu[s], cu[s+1])`` of the step (``cu`` None: row ``s``, a pure decode step); ``slots[s]`` is its
+state slot (< 0: padding row, skipped).
+"""
+
+from __future__ import annotations
+
+import dataclasses
+import math
+from typing import Optional
+
+import torch
+
+from ._dispatch import check, lib, ptr, require, stream, use_hip
+
+
+@dataclasses.dataclass
+class ScanSpec:
+    """Constants of one recurrent layer (device tensors are fp32)."""
+    heads: int
+    dim: int                        # dk
+    vdim: int                       # dv
+    mode: str                       # "decay" | "exp_gates"
+    decay: Optional[torch.Tensor] = None        # [H] fp32 ("decay")
+    cap: float = 0.0                            # gate soft cap ("exp_gates")
+    inv_freq: Optional[torch.Tensor] = None     # [rot_dims / 2] fp32
+    rot_dims: int = 0
+    rot_half: bool = True
+    qscale: float = 1.0
+    kscale: float = 1.0
+    gate_act: str = "silu"          # "silu" | "sigmoid"
+    out_scale: float = 1.0
+    eps: float = 0.0
+
+
+class ScanState:
+    """Per-sequence slots of one recurrent layer: S fp32 [slots, H, dk, dv]; with exponential
+    gates also the normaliser n [slots, H, dk] and the running maximum m [slots, H]."""
+
+    __slots__ = ("S", "n", "m")
+
+    def __init__(self, S: torch.Tensor, n: Optional[torch.Tensor] = None,
+                 m: Optional[torch.Tensor] = None):
+        self.S, self.n, self.m = S, n, m
+
+    @classmethod
+    def allocate(cls, num_slots: int, spec: ScanSpec, device):
+        z = lambda *shape: torch.zeros(*shape, dtype=torch.float32, device=device)
+        n = max(1, num_slots)
+        if spec.mode == "exp_gates":
+            return cls(z(n, spec.heads, spec.dim, spec.vdim), z(n, spec.heads, spec.dim),
+                       z(n, spec.heads))
+        return cls(z(n, spec.heads, spec.dim, spec.vdim))
+
+    @staticmethod
+    def slot_bytes(spec: ScanSpec) -> int:
+        per = spec.heads * spec.dim * spec.vdim
+        if spec.mode == "exp_gates":
+            per += spec.heads * (spec.dim + 1)
+        return 4 * per
+
+
+def _seq_bounds(cu: Optional[torch.Tensor], nseq: int):
+    if cu is None:
+        return [(s, s + 1) for s in range(nseq)]
+    c = cu.tolist()
+    return [(c[s], c[s + 1]) for s in range(nseq)]
+
+
+def _rotate(v: torch.Tensor, pos: torch.Tensor, spec: ScanSpec) -> torch.Tensor:
+    """v fp32 [T, H, D]; pos [T]."""
+    rd = spec.rot_dims
+    if not rd:
+        return v
+    ang = pos.float()[:, None] * spec.inv_freq.float()[None, :rd // 2]       # [T, rd/2]
+    cs, sn = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+    out = v.clone()
+    if spec.rot_half:
+        a, b = v[..., :rd // 2], v[..., rd // 2:rd]
+        out[..., :rd // 2], out[..., rd // 2:rd] = a * cs - b * sn, b * cs + a * sn
+    else:
+        a, b = v[..., 0:rd:2], v[..., 1:rd:2]
+        out[..., 0:rd:2], out[..., 1:rd:2] = a * cs - b * sn, b * cs + a * sn
+    return out
+
+
+def linear_scan(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int,
+                spec: ScanSpec, state: ScanState, slots: torch.Tensor,
+                cu: Optional[torch.Tensor], nseq: int, positions: torch.Tensor,
+                seq_lens: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None,
+                i_off: int = 0, f_off: int = 0, out: Optional[torch.Tensor] = None
+                ) -> torch.Tensor:
+    """fused [T, *]: rows of one fused projection holding q [H*dk], k [H*dk], v [H*dv], the gate
+    [H*dv] (and, with exponential gates, the H input-gate and H forget-gate pre-activations) at
+    the given column offsets -> y [T, H*dv] in fused's dtype (``out``: a view to write into).
+    ``norm_w`` [H*dv]: weight after the head RMS norm.  Updates the sequences' slots."""
+    T = fused.shape[0]
+    H, D, Dv = spec.heads, spec.dim, spec.vdim
+    exp_gates = spec.mode == "exp_gates"
+    if out is None:
+        out = torch.empty(T, H * Dv, dtype=fused.dtype, device=fused.device)
+    require(out.shape == (T, H * Dv) and out.dtype == fused.dtype and out.stride(1) == 1,
+            "linear_scan: out layout")
+    if not use_hip(fused):
+        f = fused.float()
+        q = _rotate(f[:, q_off:q_off + H * D].reshape(T, H, D), positions[:T], spec) * spec.qscale
+        k = _rotate(f[:, k_off:k_off + H * D].reshape(T, H, D), positions[:T], spec) * spec.kscale
+        v = f[:, v_off:v_off + H * Dv].reshape(T, H, Dv)
+        g = f[:, g_off:g_off + H * Dv]
+        y = torch.zeros(T, H, Dv)
+        if exp_gates:
+            gi = spec.cap * torch.tanh(f[:, i_off:i_off + H] / spec.cap)
+            gf = torch.nn.functional.logsigmoid(spec.cap * torch.tanh(f[:, f_off:f_off + H]
+                                                                      / spec.cap))
+        for s, (lo, hi) in enumerate(_seq_bounds(cu, nseq)):
+            sl = int(slots[s])
+            if hi <= lo or sl < 0:
+                continue
+            fresh = int(positions[lo]) == 0
+            S = torch.zeros(H, D, Dv) if fresh else state.S[sl].clone()
+            if exp_gates:
+                n = torch.zeros(H, D) if fresh else state.n[sl].clone()
+                m = torch.zeros(H) if fresh else state.m[sl].clone()
+            for t in range(lo, hi):
+                kv = k[t][:, :, None] * v[t][:, None, :]
+                if exp_gates:
+                    m_new = torch.maximum(gf[t] + m, gi[t])
+                    a, b = torch.exp(gf[t] + m - m_new), torch.exp(gi[t] - m_new)
+                    S = a[:, None, None] * S + b[:, None, None] * kv
+                    n = a[:, None] * n + b[:, None] * k[t]
+                    m = m_new
+                    den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-m)) + 1e-6
+                    o = torch.einsum("hi,hij->hj", q[t], S) / den[:, None]
+                else:
+                    S = spec.decay.float()[:, None, None] * S + kv
+                    o = torch.einsum("hi,hij->hj", q[t], S)
+                y[t] = o / torch.sqrt((o * o).mean(-1, keepdim=True) + spec.eps)
+            state.S[sl] = S
+            if exp_gates:
+                state.n[sl], state.m[sl] = n, m
+        y = y.reshape(T, H * Dv)
+        if norm_w is not None:
+            y = y * norm_w.float()
+        y = y * (torch.nn.functional.silu(g) if spec.gate_act == "silu" else torch.sigmoid(g))
+        out.copy_((y * spec.out_scale).to(out.dtype))
+        return out
+    bf = fused.dtype == torch.bfloat16
+    require(bf or fused.dtype == torch.float32, "linear_scan: bf16 or fp32")
+    require(fused.stride(1) == 1 and max(q_off + H * D, k_off + H * D, v_off + H * Dv,
+                                         g_off + H * Dv) <= fused.shape[1],
+            "linear_scan: columns outside the row")
+    require(spec.mode in ("decay", "exp_gates") and spec.gate_act in ("silu", "sigmoid"),
+            "linear_scan: mode")
+    require(state.S.dtype == torch.float32 and state.S.is_contiguous() and
+            state.S.shape[1:] == (H, D, Dv), "linear_scan: state layout")
+    if exp_gates:
+        require(max(i_off, f_off) + H <= fused.shape[1] and state.n is not None and
+                state.m is not None and state.n.is_contiguous() and state.m.is_contiguous() and
+                spec.cap > 0, "linear_scan: gates")
+    else:
+        require(spec.decay is not None and spec.decay.dtype == torch.float32 and
+                spec.decay.is_cuda and spec.decay.numel() == H, "linear_scan: decay per head")
+    require(spec.rot_dims == 0 or (spec.inv_freq is not None and spec.inv_freq.is_cuda and
+                                   spec.inv_freq.dtype == torch.float32 and
+                                   spec.inv_freq.numel() >= spec.rot_dims // 2 and
+                                   spec.rot_dims <= D and spec.rot_dims % 2 == 0),
+            "linear_scan: rotation")
+    require(slots.dtype == torch.int32 and positions.dtype == torch.int32 and
+            (cu is None or cu.dtype == torch.int32), "linear_scan: int32 metadata")
+    require(norm_w is None or (norm_w.dtype == fused.dtype and norm_w.is_contiguous() and
+                               norm_w.numel() == H * Dv), "linear_scan: norm weight")
+    check(lib().eia_linear_scan(
+        ptr(fused), fused.stride(0), q_off, k_off, v_off, g_off, i_off, f_off, ptr(spec.decay),
+        ptr(spec.inv_freq), spec.rot_dims, 1 if spec.rot_half else 0, float(spec.qscale),
+        float(spec.kscale), float(spec.cap), float(spec.out_scale), ptr(norm_w), ptr(state.S),
+        ptr(state.n), ptr(state.m), ptr(slots), ptr(cu), ptr(positions), ptr(seq_lens), ptr(out),
+        out.stride(0), float(spec.eps), nseq, H, D, Dv, 1 if exp_gates else 0,
+        0 if spec.gate_act == "silu" else 1, 1 if bf else 0, stream(fused)), "linear_scan")
+    return out

@@ -336,44 +336,80 @@ UNGATED_SMALL_EXPERT = int(os.environ.get("EIA_UNGATED_SMALL_EXPERT", str(2 * 10
 def route_grouped(x: torch.Tensor, router_w: torch.Tensor, k: int, num_groups: int,
                   keep_groups: int, route_scale: float,
                   row_len: Optional[torch.Tensor] = None,
-                  always_on: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Group-limited sigmoid routing (moe.hip route_grouped_kernel): fp32 logits x W_r^T,
-    scores = sigmoid; experts form ``num_groups`` equal groups of neighbours, a group scores the
-    sum of its two largest scores, only the ``keep_groups`` best groups are eligible, the ``k``
-    largest eligible scores win and weigh score * route_scale (not renormalised; ties to the
-    lower index).  -> (weights fp32 [T, k], expert ids int32 [T, k]).
+                  always_on: bool = False, *, scoring: str = "sigmoid", group_score: str = "top2",
+                  correction: Optional[torch.Tensor] = None, identity: int = 0,
+                  gate_w: Optional[torch.Tensor] = None):
+    """Group-limited routing (moe.hip route_grouped_kernel): fp32 logits x W_r^T; scores =
+    sigmoid, or softmax over all outputs (``scoring``); the outputs form ``num_groups`` equal
+    groups of neighbours; selection ranks the choice scores ``score + correction`` (fp32 [E],
+    optional; they may be negative), a group scores the sum of its two largest choice scores
+    (``group_score`` "top2") or the largest ("max"), only the ``keep_groups`` best groups are
+    eligible, the ``k`` largest eligible choice scores win and weigh score * route_scale (the
+    plain score; not renormalised; ties to the lower index).
+    -> (weights fp32 [T, k], ids int32 [T, k]).
     ``always_on``: one more column per token naming expert E with weight 1 -- an always-on
     (shared) expert whose weights are stored behind the E routed ones, so that it rides in the
-    same grouped launches."""
+    same grouped launches.
+    ``identity``: the last that many router outputs are identity experts (no weights; their
+    output is the token's input); their ids (>= E - identity) are reported like the others.
+    ``gate_w`` [1, H] or [H]: one more dot product per token, for the gate of a shared expert.
+    With ``identity`` or ``gate_w`` the result is (weights, ids, ident_w, gate): the summed
+    weight of a token's chosen identity experts fp32 [T] (None without identity experts) and
+    sigmoid(gate_w . x) fp32 [T] (None without gate_w)."""
     T, H = x.shape
     E = router_w.shape[0]
     ko = k + (1 if always_on else 0)
+    n_real = E - int(identity)
+    more = bool(identity) or gate_w is not None
     if not use_hip(x):
-        s = torch.sigmoid(x.float() @ router_w.float().t())
+        z = x.float() @ router_w.float().t()
+        s = torch.sigmoid(z) if scoring == "sigmoid" else torch.softmax(z, -1)
+        c = s + correction.float() if correction is not None else s
         per = E // num_groups
-        gs = s.view(T, num_groups, per).topk(min(2, per), -1).values.sum(-1)
+        gs = c.view(T, num_groups, per).topk(min(2 if group_score == "top2" else 1, per), -1
+                                             ).values.sum(-1)
         # stable descending order: ties keep the lower index
         gi = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep_groups]
         ok = torch.zeros(T, num_groups, dtype=torch.bool)
         ok.scatter_(1, gi, True)
-        masked = torch.where(ok[:, :, None].expand(T, num_groups, per).reshape(T, E), s,
-                             torch.full_like(s, -1.0))
+        masked = torch.where(ok[:, :, None].expand(T, num_groups, per).reshape(T, E), c,
+                             torch.full_like(c, float("-inf")))
         order = torch.sort(masked, dim=-1, descending=True, stable=True).indices[:, :k]
         w, ids = s.gather(1, order) * route_scale, order.to(torch.int32)
+        if row_len is not None:
+            padr = row_len[:T] == 0
+            w = torch.where(padr[:, None], torch.zeros_like(w), w)
+            ids = torch.where(padr[:, None], torch.full_like(ids, E), ids)
+        iw = (w * (ids >= n_real)).sum(-1) if identity else None
         if always_on:
             w = torch.cat([w, torch.ones(T, 1)], 1)
             ids = torch.cat([ids, torch.full((T, 1), E, dtype=torch.int32)], 1)
-        return w, ids
+        if not more:
+            return w, ids
+        g = torch.sigmoid(x.float() @ gate_w.float().reshape(-1)) if gate_w is not None else None
+        return w, ids, iw, g
     require(x.stride(1) == 1 and router_w.is_contiguous() and router_w.dtype == x.dtype and
             x.dtype in (torch.bfloat16, torch.float32), "route_grouped: layout")
+    require(scoring in ("sigmoid", "softmax") and group_score in ("top2", "max"),
+            "route_grouped: scoring / group score")
+    require(correction is None or (correction.dtype == torch.float32 and correction.is_cuda and
+                                   correction.is_contiguous() and correction.numel() == E),
+            "route_grouped: fp32 correction per output")
+    require(gate_w is None or (gate_w.dtype == x.dtype and gate_w.is_contiguous() and
+                               gate_w.numel() == H), "route_grouped: gate row")
     w = torch.empty(T, ko, dtype=torch.float32, device=x.device)
     ids = torch.empty(T, ko, dtype=torch.int32, device=x.device)
+    iw = torch.empty(T, dtype=torch.float32, device=x.device) if identity else None
+    g = torch.empty(T, dtype=torch.float32, device=x.device) if gate_w is not None else None
     check(lib().eia_moe_route_grouped(ptr(x), x.stride(0), ptr(router_w), H, T, E, k, num_groups,
                                       keep_groups, float(route_scale), ptr(w), ptr(ids),
                                       ptr(row_len), 1 if always_on else 0,
                                       1 if x.dtype == torch.bfloat16 else 0,
-                                      stream(x)), "moe_route_grouped")
-    return w, ids
+                                      1 if scoring == "softmax" else 0,
+                                      1 if group_score == "max" else 0, ptr(correction), n_real,
+                                      ptr(iw), ptr(gate_w), ptr(g), stream(x)),
+          "moe_route_grouped")
+    return (w, ids, iw, g) if more else (w, ids)
 
 
 def ungated_moe(x: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, topk_w: torch.Tensor,
@@ -496,3 +532,15 @@ def combine_post_norm(h2: torch.Tensor, topk_w: torch.Tensor, inv: torch.Tensor,
         shared.stride(0) if shared is not None else 0, ptr(norm_w), float(eps), ptr(x), ptr(xb),
         W, T, W, 1 if bf else 0, stream(h2)), "moe_combine_postnorm")
     return xb if bf else (x if copy else None)
+
+
+def finish_gated(routed: torch.Tensor, x: torch.Tensor, ident_w: Optional[torch.Tensor],
+                 shared: Optional[torch.Tensor], sgate: Optional[torch.Tensor]) -> torch.Tensor:
+    """End of an expert block with identity experts and a gated shared expert, summed in fp32:
+    routed + ident_w[:, None] * x + sgate[:, None] * shared  -> [T, H] in x's dtype."""
+    y = routed.float()
+    if ident_w is not None:
+        y = y + ident_w[:, None] * x.float()
+    if shared is not None:
+        y = y + (shared.float() * sgate[:, None] if sgate is not None else shared.float())
+    return y.to(x.dtype)

@@ -234,3 +234,66 @@ def residual_rms_step(x: torch.Tensor, eps: float, ys=(), w_next: Optional[torch
                             ptr(x), ptr(w_next), ptr(h), W, float(eps), T, W,
                             1 if dt == torch.bfloat16 else 0, stream(x)), "add_rms")
     return h
+
+
+def hyper_step(X: torch.Tensor, eps: float, y=None, mix: Optional[torch.Tensor] = None,
+               outw: Optional[torch.Tensor] = None, ymult: float = 1.0,
+               in_next: Optional[torch.Tensor] = None, w_next: Optional[torch.Tensor] = None,
+               w_offset: float = 0.0) -> Optional[torch.Tensor]:
+    """Boundary of a sublayer whose residual is kept as several streams joined by
+    hyper-connections, X fp32 [T, NS, W] updated in place, in one pass over the row:
+
+        X_j <- sum_s mix[s, j] X_s + ymult * outw[j] * y        (y given; all streams at once)
+        u    = sum_j in_next[j] X_j
+        h    = u / sqrt(mean(u^2) + eps) * (w_offset + w_next)   (w_next given: returned)
+
+    ``mix`` [NS, NS] (from, to), ``outw`` [NS] and ``in_next`` [NS] are fp32.  y is a tensor in the
+    activation dtype or a ``gemm.SplitK`` (fp32 partial sums of the GEMM that produced it, plus
+    its bias), reduced here.  NS = 1 with unit constants is the plain residual sum."""
+    from .gemm import SplitK
+    T, NS, W = X.shape
+    split = isinstance(y, SplitK)
+    if split and (not use_hip(X)):
+        y = y.part.sum(0) + (y.bias.float() if y.bias is not None else 0.0)
+        split = False
+    if not use_hip(X):
+        if y is not None:
+            X.copy_(torch.einsum("sj,tsw->tjw", mix.float(), X)
+                    + ymult * outw.float()[None, :, None] * y.float()[:, None, :])
+        if w_next is None:
+            return None
+        u = torch.einsum("j,tjw->tw", in_next.float(), X)
+        return (u / torch.sqrt((u * u).mean(-1, keepdim=True) + eps)
+                * (w_offset + w_next.float())).to(w_next.dtype)
+    require(X.dtype == torch.float32 and X.is_contiguous() and NS <= 8, "hyper_step: fp32 streams")
+    dt = w_next.dtype if w_next is not None else (
+        (y.bias.dtype if y.bias is not None else torch.bfloat16) if split else
+        (y.dtype if y is not None else torch.float32))
+    require(dt in (torch.bfloat16, torch.float32), "hyper_step: bf16 or fp32")
+    for t in (mix, outw, in_next):
+        require(t is None or (t.dtype == torch.float32 and t.is_cuda and t.is_contiguous()),
+                "hyper_step: fp32 device constants")
+    yt = part = ybias = None
+    sk = 0
+    if split:
+        require(y.M == T and y.N == W and y.part.is_contiguous() and
+                y.part.dtype == torch.float32 and (y.bias is None or y.bias.dtype == dt),
+                "hyper_step: partials")
+        part, sk, ybias = y.part, y.sk, y.bias
+    elif y is not None:
+        require(y.shape == (T, W) and y.stride(-1) == 1 and y.dtype == dt, "hyper_step: y layout")
+        yt = y
+    if y is not None:
+        require(mix is not None and outw is not None and mix.numel() == NS * NS and
+                outw.numel() == NS, "hyper_step: stream constants")
+    h = None
+    if w_next is not None:
+        require(w_next.numel() == W and in_next is not None and in_next.numel() == NS,
+                "hyper_step: next norm")
+        h = torch.empty(T, W, dtype=dt, device=X.device)
+    check(lib().eia_hyper_step(ptr(X), NS, W, ptr(yt), yt.stride(0) if yt is not None else 0,
+                               ptr(part), sk, ptr(ybias), ptr(mix), ptr(outw), float(ymult),
+                               ptr(in_next), ptr(w_next), float(w_offset), ptr(h),
+                               h.stride(0) if h is not None else 0, float(eps), T,
+                               1 if dt == torch.bfloat16 else 0, stream(X)), "hyper_step")
+    return h

@@ -74,13 +74,16 @@ def rotary_frequencies(dims: int, base: float, scaling: Optional[dict] = None, d
     multiplied by amp.  f_i = base^(-2i/dims); with ``scaling`` = {factor, original, fast, slow}
     (YaRN) the pairs that turn fewer than ``slow`` times over ``original`` positions are slowed
     by ``factor``, those that turn more than ``fast`` times keep their frequency, the ones
-    between are blended linearly in the pair index, and amp = 0.1 ln(factor) + 1.  Evaluated in
-    float64 and rounded once."""
+    between are blended linearly in the pair index, and amp = 0.1 ln(factor) + 1.  A ``scaling``
+    that gives only ``factor`` is linear position interpolation: every f_i is divided by it.
+    Evaluated in float64 and rounded once."""
     import math
     i = torch.arange(dims // 2, dtype=torch.float64)
     f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(dims, 1))
     amp = 1.0
-    if scaling:
+    if scaling and "original" not in scaling:
+        f = f / float(scaling["factor"])
+    elif scaling:
         factor, orig = float(scaling["factor"]), float(scaling["original"])
 
         def pair_of(turns: float) -> float:       # the (real-valued) pair index turning that often

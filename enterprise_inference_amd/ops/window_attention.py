@@ -8,9 +8,10 @@ map ``h*P + c`` reads key map ``(h // (H//G))*P + c`` and value head ``h // (H//
 the score of (query position i, key j) is ``(q.k) * mult[m] - slope[m]*(i-j)``, optionally mixed
 across maps by a matrix (``talk``), masked to ``j <= i and (i-j < window or j < keep)`` and
 soft-maxed -- or, with ``spec.weights`` 1, every visible key simply weighs
-``sigmoid(score + bias[m])`` and nothing is normalised over the keys.  ``spec.epilogue`` 0
-multiplies the heads by ``sigmoid(gate)``; 1 combines a head's two maps as ``a1 - lam*a2``,
-divides by the root mean square over the head and scales.
+``sigmoid(score + bias[m])`` and nothing is normalised over the keys.  With ``spec.sink`` the
+softmax denominator of map m also holds ``exp(sink[m])``, a term without key or value.
+``spec.epilogue`` 0 multiplies the heads by ``sigmoid(gate)`` and by ``spec.post``; 1 combines
+a head's two maps as ``a1 - lam*a2``, divides by the root mean square over the head and scales.
 
 A step's rows are [decode rows (1 per sequence) | prefill chunks]; both parts read the cache
 after ``qk_norm_cache`` wrote this step's rows, so chunked prompts need no special path.
@@ -50,6 +51,7 @@ class WindowSpec:
     post: float = 1.0
     weights: int = 0                # 0: softmax over the visible keys; 1: sigmoid(score + bias)
     bias: Optional[torch.Tensor] = None     # [H*P], added to the score inside the sigmoid
+    sink: Optional[torch.Tensor] = None     # [H*P], exp(sink) joins the softmax denominator
 
 
 def build_work(q_lens: List[int], qblock: int) -> List[int]:
@@ -267,12 +269,14 @@ def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpe
             sc = spec.talk @ sc
         if spec.weights == 1:
             w = torch.sigmoid(sc + (spec.bias[:, None] if spec.bias is not None else 0.0))
+        elif spec.sink is not None:
+            w = torch.softmax(torch.cat([sc, spec.sink[:, None]], -1), -1)[:, :-1]
         else:
             w = torch.softmax(sc, -1)
         w = w.view(H, P, len(js))
         a = torch.einsum("hpn,nhd->hpd", w, vals)
         if spec.epilogue == 0:
-            o = a[:, 0].reshape(H * Dv)
+            o = a[:, 0].reshape(H * Dv) * spec.post
             if gate is not None:
                 o = o * torch.sigmoid(gate[row].float())
         else:
@@ -283,13 +287,18 @@ def _ref_rows(q, k_cache, v_cache, block_table, positions, gate, spec: WindowSpe
 
 
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, md,
-                     spec: WindowSpec, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     spec: WindowSpec, gate: Optional[torch.Tensor] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """q [T, H*P*D] (normed; contiguous last dim), gate [T, H*Dv] before the sigmoid or None ->
-    [T, H*Dv] in q's dtype.  ``md`` is the step's AttentionMetadata."""
+    [T, H*Dv] in q's dtype.  ``md`` is the step's AttentionMetadata.  ``out``: a [T, H*Dv] view
+    (contiguous last dim; the columns of a wider row that another mixer shares) to write into."""
     T = q.shape[0]
     H, P, D, Dv = spec.heads, spec.maps, spec.dim, spec.vdim
     nd = md.num_decode
-    out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    if out is None:
+        out = torch.empty(T, H * Dv, dtype=q.dtype, device=q.device)
+    require(out.shape == (T, H * Dv) and out.dtype == q.dtype and out.stride(1) == 1,
+            "window_attention: out layout")
     if not use_hip(q, k_cache):
         if nd:
             out[:nd] = _ref_rows(q[:nd], k_cache, v_cache, md.decode_block_tables,
@@ -314,7 +323,8 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     require(md.positions.dtype == torch.int32, "positions int32")
     require(spec.weights in (0, 1) and (spec.weights == 0 or (spec.talk is None and P == 1)),
             "window_attention: sigmoid weights come without head mixing or map pairs")
-    for t in (spec.mult, spec.slope, spec.talk, spec.lam, spec.bias):
+    require(spec.sink is None or spec.weights == 0, "window_attention: a sink needs softmax weights")
+    for t in (spec.mult, spec.slope, spec.talk, spec.lam, spec.bias, spec.sink):
         require(t is None or (t.dtype == torch.float32 and t.is_cuda and t.is_contiguous()),
                 "window_attention: fp32 device constants")
     bs = k_cache.shape[1]
@@ -339,7 +349,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                 ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0,
                 ptr(o), o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep,
                 spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), spec.weights,
-                ptr(spec.bias), NP, ptr(pa), ptr(pm), stream(q)), "window_attn_mfma")
+                ptr(spec.bias), NP, ptr(pa), ptr(pm), ptr(spec.sink), stream(q)), "window_attn_mfma")
             return
         check(lib().eia_window_attn(
             ptr(qa), qa.stride(0), ptr(k_cache), ptr(v_cache), ptr(bt), bt.stride(0),
@@ -347,7 +357,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             ptr(spec.slope), ptr(spec.talk), ptr(g), g.stride(0) if g is not None else 0, ptr(o),
             o.stride(0), H, spec.kv_heads, P, D, Dv, bs, spec.window, spec.keep, qb,
             spec.epilogue, ptr(spec.lam), float(spec.eps), float(spec.post), spec.weights,
-            ptr(spec.bias), 1 if bf else 0, stream(q)), "window_attn")
+            ptr(spec.bias), ptr(spec.sink), 1 if bf else 0, stream(q)), "window_attn")
 
     if nd:
         launch(0, nd, md.decode_block_tables, md.decode_seq_lens, None, None, 1)
