@@ -24,7 +24,9 @@ def act_and_mul(x, act: str = "silu") -> torch.Tensor:
                                                kind, stream(out)), "splitk_act_and_mul")
             return out
         x = x.materialize()
-    if not (use_hip(x) and x.dtype == torch.bfloat16):
+    # (the kernel works on 16-byte units: other widths take the unfused form)
+    if not (use_hip(x) and x.dtype == torch.bfloat16 and x.shape[-1] % 16 == 0
+            and x.stride(-1) == 1):
         return ref.silu_and_mul(x) if kind == 0 else ref.gelu_and_mul(x) if kind == 1 else (
             (torch.nn.functional.gelu(x[..., :x.shape[-1] // 2].float()) *
              x[..., x.shape[-1] // 2:].float()).to(x.dtype))
