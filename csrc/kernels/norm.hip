@@ -507,7 +507,8 @@ EIA_API int eia_add_rms(const void* y1, long ld1, const float* p1, int sk1, cons
 // arrays.  NS = 1 with mix = outw = in_next = 1 is the plain residual sum.  All arithmetic fp32.
 constexpr int HC_MAX = 8;
 
-template <typename T>
+// V: columns per thread and step (4: 16-byte accesses; needs W, ldy and ldh multiples of 4)
+template <typename T, int V>
 __global__ void __launch_bounds__(256)
 hyper_step_kernel(float* __restrict__ X, int NS, int W, const T* __restrict__ y, long ldy,
                   const float* __restrict__ part, int sk, long pstride,
@@ -529,45 +530,92 @@ hyper_step_kernel(float* __restrict__ X, int NS, int W, const T* __restrict__ y,
     for (int j = 0; j < HC_MAX; ++j) mx[s][j] = (upd && s < NS && j < NS) ? mix[s * NS + j] : 0.f;
   }
   float ss = 0.f;
-  for (int c = threadIdx.x; c < W; c += blockDim.x) {
-    float xs[HC_MAX];
+  for (int c = V * threadIdx.x; c < W; c += V * blockDim.x) {
+    float xs[HC_MAX][V];
 #pragma unroll
-    for (int s = 0; s < HC_MAX; ++s) xs[s] = s < NS ? xr[(long)s * W + c] : 0.f;
-    if (upd) {
-      float yv;
-      if (y) {
-        yv = ld_f32<T>(y + row * ldy, c);
+    for (int s = 0; s < HC_MAX; ++s) {
+      if (s < NS) {
+        if constexpr (V == 4) {
+          const f32x4 v = *reinterpret_cast<const f32x4*>(xr + (long)s * W + c);
+#pragma unroll
+          for (int e = 0; e < V; ++e) xs[s][e] = v[e];
+        } else {
+          xs[s][0] = xr[(long)s * W + c];
+        }
       } else {
-        yv = ybias ? ld_f32<T>(ybias, c) : 0.f;
+#pragma unroll
+        for (int e = 0; e < V; ++e) xs[s][e] = 0.f;
+      }
+    }
+    if (upd) {
+      float yv[V];
+      if (y) {
+        if constexpr (V == 4) {
+          const f32x4 v = ld4_f32<T>(y + row * ldy + c);
+#pragma unroll
+          for (int e = 0; e < V; ++e) yv[e] = v[e];
+        } else {
+          yv[0] = ld_f32<T>(y + row * ldy, c);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < V; ++e) yv[e] = ybias ? ld_f32<T>(ybias, c + e) : 0.f;
         const float* p = part + row * (long)W + c;
-        for (int z = 0; z < sk; ++z) yv += p[z * pstride];
+        for (int z = 0; z < sk; ++z) {
+          if constexpr (V == 4) {
+            const f32x4 v = *reinterpret_cast<const f32x4*>(p + z * pstride);
+#pragma unroll
+            for (int e = 0; e < V; ++e) yv[e] += v[e];
+          } else {
+            yv[0] += p[z * pstride];
+          }
+        }
       }
-      float nx[HC_MAX];
+      float nx[HC_MAX][V];
+#pragma unroll
+      for (int j = 0; j < HC_MAX; ++j)
+#pragma unroll
+        for (int e = 0; e < V; ++e) {
+          float v = ow[j] * yv[e];
+#pragma unroll
+          for (int s = 0; s < HC_MAX; ++s) v += mx[s][j] * xs[s][e];
+          nx[j][e] = v;
+        }
 #pragma unroll
       for (int j = 0; j < HC_MAX; ++j) {
-        float v = ow[j] * yv;
+        if (j < NS) {
+          if constexpr (V == 4)
+            *reinterpret_cast<f32x4*>(xr + (long)j * W + c) =
+                f32x4{nx[j][0], nx[j][1], nx[j][2], nx[j][3]};
+          else
+            xr[(long)j * W + c] = nx[j][0];
+        }
 #pragma unroll
-        for (int s = 0; s < HC_MAX; ++s) v += mx[s][j] * xs[s];
-        nx[j] = v;
-      }
-#pragma unroll
-      for (int j = 0; j < HC_MAX; ++j) {
-        if (j < NS) xr[(long)j * W + c] = nx[j];
-        xs[j] = nx[j];
+        for (int e = 0; e < V; ++e) xs[j][e] = nx[j][e];
       }
     }
     if (h) {
-      float u = 0.f;
 #pragma unroll
-      for (int j = 0; j < HC_MAX; ++j) u += iw[j] * xs[j];
-      u_s[c] = u;
-      ss += u * u;
+      for (int e = 0; e < V; ++e) {
+        float u = 0.f;
+#pragma unroll
+        for (int j = 0; j < HC_MAX; ++j) u += iw[j] * xs[j][e];
+        u_s[c + e] = u;
+        ss += u * u;
+      }
     }
   }
   if (!h) return;
   const float inv = 1.0f / sqrtf(block_sum(ss, scratch) / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += blockDim.x)
-    st_f32<T>(h + row * ldh, c, u_s[c] * inv * (w_off + ld_f32<T>(w_next, c)));
+  for (int c = V * threadIdx.x; c < W; c += V * blockDim.x) {
+    if constexpr (V == 4) {
+      const f32x4 wv = ld4_f32<T>(w_next + c);
+      const f32x4 u = *reinterpret_cast<const f32x4*>(u_s + c);
+      st4_f32<T>(h + row * ldh + c, u * inv * (wv + w_off));
+    } else {
+      st_f32<T>(h + row * ldh, c, u_s[c] * inv * (w_off + ld_f32<T>(w_next, c)));
+    }
+  }
 }
 
 // X fp32 [rows, NS, W] contiguous; y, ybias, w_next and h are bf16 when is_bf16 else fp32.
@@ -580,16 +628,19 @@ EIA_API int eia_hyper_step(float* X, int NS, int W, const void* y, long ldy, con
     return EIA_BAD_SHAPE;
   if ((size_t)W * sizeof(float) > 64 * 1024) return EIA_UNSUPPORTED;
   if (rows == 0) return EIA_OK;
+  const bool vec = W % 4 == 0 && ldy % 4 == 0 && ldh % 4 == 0;
   const int threads = W >= 1024 ? 256 : (W >= 512 ? 128 : 64);
   const size_t lds = h ? sizeof(float) * W : 0;
   const long ps = (long)rows * W;
-  if (is_bf16)
-    hipLaunchKernelGGL((hyper_step_kernel<bf16_t>), dim3(rows), dim3(threads), lds, st, X, NS, W,
-                       (const bf16_t*)y, ldy, part, sk, ps, (const bf16_t*)ybias, mix, outw, ymult,
-                       in_next, (const bf16_t*)w_next, w_off, (bf16_t*)h, ldh, eps);
-  else
-    hipLaunchKernelGGL((hyper_step_kernel<float>), dim3(rows), dim3(threads), lds, st, X, NS, W,
-                       (const float*)y, ldy, part, sk, ps, (const float*)ybias, mix, outw, ymult,
-                       in_next, (const float*)w_next, w_off, (float*)h, ldh, eps);
+#define HC_LAUNCH(TT, VV)                                                                        \
+  hipLaunchKernelGGL((hyper_step_kernel<TT, VV>), dim3(rows), dim3(threads), lds, st, X, NS, W,  \
+                     (const TT*)y, ldy, part, sk, ps, (const TT*)ybias, mix, outw, ymult,        \
+                     in_next, (const TT*)w_next, w_off, (TT*)h, ldh, eps)
+  if (is_bf16) {
+    if (vec) HC_LAUNCH(bf16_t, 4); else HC_LAUNCH(bf16_t, 1);
+  } else {
+    if (vec) HC_LAUNCH(float, 4); else HC_LAUNCH(float, 1);
+  }
+#undef HC_LAUNCH
   EIA_LAUNCH_CHECK();
 }

@@ -127,7 +127,6 @@ class DaburaxForCausalLM(nn.Module):
     supports_pp = False
     supports_float32 = True        # every kernel of this model has an fp32 form
     needs_state_slots = True       # recurrent layers and the previous token of the bigram term
-    supports_graphs = False        # the expert block reads row offsets back on some shapes
 
     def __init__(self, cfg: ModelConfig, dtype=torch.bfloat16, device=None):
         super().__init__()
@@ -153,6 +152,11 @@ class DaburaxForCausalLM(nn.Module):
         self.final_norm = _plain((W,), dtype, device)
         self.head = _plain((cfg.vocab_size, W), dtype, device)
         self.ones = torch.ones(max(1, self.streams), dtype=torch.float32, device=device)
+        # decode steps replay HIP graphs when every expert block has a device-side grouped form
+        # (bf16, width a multiple of 128 and expert ff a multiple of 64); else they read row
+        # offsets back per layer
+        self.supports_graphs = dtype == torch.bfloat16 and all(
+            L.mlp is None or (W % 128 == 0 and L.mlp.I % 64 == 0) for L in self.layers)
         # the sublayer boundaries in order: (layer, hyper-connection, norm weight)
         self.steps = [(i, hc, w) for i, L in enumerate(self.layers) for hc, w in L.boundaries()]
 

@@ -536,11 +536,28 @@ def combine_post_norm(h2: torch.Tensor, topk_w: torch.Tensor, inv: torch.Tensor,
 
 def finish_gated(routed: torch.Tensor, x: torch.Tensor, ident_w: Optional[torch.Tensor],
                  shared: Optional[torch.Tensor], sgate: Optional[torch.Tensor]) -> torch.Tensor:
-    """End of an expert block with identity experts and a gated shared expert, summed in fp32:
+    """End of an expert block with identity experts and a gated shared expert, summed in fp32
+    (moe.hip moe_finish_kernel, one launch):
     routed + ident_w[:, None] * x + sgate[:, None] * shared  -> [T, H] in x's dtype."""
-    y = routed.float()
-    if ident_w is not None:
-        y = y + ident_w[:, None] * x.float()
-    if shared is not None:
-        y = y + (shared.float() * sgate[:, None] if sgate is not None else shared.float())
-    return y.to(x.dtype)
+    if not use_hip(x):
+        y = routed.float()
+        if ident_w is not None:
+            y = y + ident_w[:, None] * x.float()
+        if shared is not None:
+            y = y + (shared.float() * sgate[:, None] if sgate is not None else shared.float())
+        return y.to(x.dtype)
+    T, H = x.shape
+    dt = x.dtype
+    require(dt in (torch.bfloat16, torch.float32) and routed.dtype == dt and
+            routed.shape == (T, H) and routed.stride(1) == 1 and x.stride(1) == 1 and
+            (shared is None or (shared.dtype == dt and shared.shape == (T, H) and
+                                shared.stride(1) == 1)), "finish_gated: layout")
+    for t in (ident_w, sgate):
+        require(t is None or (t.dtype == torch.float32 and t.is_contiguous() and t.numel() == T),
+                "finish_gated: fp32 per-token weights")
+    out = torch.empty(T, H, dtype=dt, device=x.device)
+    check(lib().eia_moe_finish(ptr(routed), routed.stride(0), ptr(x), x.stride(0), ptr(ident_w),
+                               ptr(shared), shared.stride(0) if shared is not None else 0,
+                               ptr(sgate), ptr(out), out.stride(0), T, H,
+                               1 if dt == torch.bfloat16 else 0, stream(x)), "moe_finish")
+    return out
