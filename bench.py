@@ -67,13 +67,16 @@ def parse():
     ap.add_argument("--mode", default="endpoint", choices=["endpoint", "engine", "design"],
                     help="design: prefill / decode throughput of a layer-list design beside the "
                          "closest existing decoder at equal layer sizes (benchmarks/design_bench.py)")
-    ap.add_argument("--design", default="sekolorn", choices=["sekolorn", "vedadra", "gapidra"],
-                    help="design mode: sekolorn beside a Mixtral-style decoder, or vedadra / gapidra "
-                         "beside a Mistral-style decoder (sliding-window GQA attention + gated MLP)")
+    ap.add_argument("--design", default="sekolorn",
+                    choices=["sekolorn", "vedadra", "gapidra", "daburax"],
+                    help="design mode: sekolorn beside a Mixtral-style decoder, vedadra / gapidra "
+                         "beside a Mistral-style decoder (sliding-window GQA attention + gated "
+                         "MLP), or daburax beside sekolorn")
     ap.add_argument("--design-sizes", default=None,
                     help="comma list; sekolorn: s, s6 (m, l: gated), default s,s6; "
-                         "vedadra: vs, vm, default vs,vm; gapidra: gs, gm, default gs,gm")
-    ap.add_argument("--design-models", default="sekolorn,mixtral,vedadra,mistral,gapidra",
+                         "vedadra: vs, vm, default vs,vm; gapidra: gs, gm, default gs,gm; "
+                         "daburax: ds, dm, default ds,dm")
+    ap.add_argument("--design-models", default="sekolorn,mixtral,vedadra,mistral,gapidra,daburax",
                     help="which of the two engines to run (profiling one of them alone)")
     ap.add_argument("--design-kernels", action="store_true",
                     help="design mode: time the design's attention / scan kernels beside the "

@@ -13,6 +13,11 @@ count, head size, window and ff.
 ``--design gapidra`` runs the Gapidra design (parallel sublayers on one norm; sigmoid window
 attention and windowed latent attention with sinks, alternating; ungated xIELU feed-forward)
 beside the same Mistral-style decoder at equal width, depth, heads, head size, window and ff.
+``--design daburax`` runs the Daburax design (hyper-connected residual streams; retention layers
+and parallel layers of sink attention beside a gated matrix memory; a group-limited mixture of
+gated experts with identity experts and a gated shared expert) beside Sekolorn, the closest
+existing design (recurrent and attention layers on state slots and paged rows, a group-routed
+mixture of experts with a shared expert), at equal width, depth, heads, experts and expert ff.
 Prefill: ``--design-prompts`` prompts of ``--design-prompt-len`` tokens, one sampled token each.
 Decode: ``--design-users`` sequences of 128 prompt tokens generating ``--design-gen`` tokens; the
 decode rate is the extra tokens over the extra time against the same run with one token.
@@ -133,6 +138,44 @@ def gapidra_config(z: dict) -> dict:
             "layers": [att, lat, lat, att, lat, att]}
 
 
+DSIZES = {
+    # name: width, heads, head dim, experts (+ 2 identity outputs), expert ff, streams, vocab
+    "ds": dict(width=1024, layers=6, heads=8, dim=128, experts=8, top=2, ff=512, streams=4,
+               vocab=32000),
+    "dm": dict(width=2048, layers=6, heads=16, dim=128, experts=16, top=2, ff=1024, streams=4,
+               vocab=32000),
+}
+
+
+def daburax_config(z: dict) -> dict:
+    H, D = z["heads"], z["dim"]
+    mlp = {"kind": "moe", "expert": {"ff": z["ff"]}, "shared": {"ff": z["ff"]},
+           "router": {"experts": z["experts"] - 2, "identity": 2, "top": z["top"],
+                      "groups": {"count": 4, "keep": 2}}}
+    ret = {"type": "retention", "mlp": mlp,
+           "mixer": {"heads": H, "dim": D, "vdim": D, "rot": {"base": 1e6, "dims": D},
+                     "decay": [1.0 - 2.0 ** (-5 - 4 * i / H) for i in range(H)]}}
+    par = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": {"heads": H, "kv_heads": max(1, H // 4), "dim": D, "vdim": D,
+                              "scale": D ** -0.5,
+                              "rot": {"base": 5e4, "dims": D // 2, "scaling": {"factor": 2.0}}},
+                     "right": {"heads": H // 2, "dim": D, "vdim": D, "gate_cap": 12.0},
+                     "left_scale": 1.0, "right_scale": 1.0}}
+    return {"architecture": "Daburax", "vocab": z["vocab"], "width": z["width"],
+            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "streams": z["streams"],
+            "embedding": {"scale": z["width"] ** 0.5,
+                          "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "layers": [ret, ret, par] * (z["layers"] // 3)}
+
+
+def sekolorn_like(z: dict) -> dict:
+    """Sekolorn at a Daburax size: same width, depth, heads, experts, top-k and expert ff."""
+    return sekolorn_config(dict(width=z["width"], layers=z["layers"], heads=z["heads"], dim=64,
+                                rot=32, kv_rank=z["width"] // 8, q_rank=z["width"] // 4,
+                                wkv_heads=z["width"] // 64, experts=z["experts"], top=z["top"],
+                                groups=4, keep=2, ff=z["ff"], vocab=z["vocab"]))
+
+
 def _measure(cfg_dict: dict, a) -> dict:
     import torch
 
@@ -184,12 +227,15 @@ def run(a) -> int:
     rows = []
     design = getattr(a, "design", "sekolorn")
     vedadra = design == "vedadra"
-    default = {"vedadra": "vs,vm", "gapidra": "gs,gm"}.get(design, "s,s6")
+    default = {"vedadra": "vs,vm", "gapidra": "gs,gm", "daburax": "ds,dm"}.get(design, "s,s6")
     for name in (a.design_sizes or default).split(","):
         if name in GATED:
             raise SystemExit(f"design size {name!r} is switched off (see GATED in "
                              "benchmarks/design_bench.py); run s or s6")
-        if design == "gapidra":
+        if design == "daburax":
+            z = DSIZES[name]
+            pair = (("Daburax", daburax_config(z)), ("Sekolorn", sekolorn_like(z)))
+        elif design == "gapidra":
             z = dict(GSIZES[name], layers=6)
             pair = (("Gapidra", gapidra_config(z)), ("Mistral-style", mistral_config(z)))
         elif vedadra:
@@ -239,6 +285,8 @@ def kernel_rates(a) -> int:
         return window_kernel_rates(a)
     if getattr(a, "design", "sekolorn") == "gapidra":
         return gapidra_kernel_rates(a)
+    if getattr(a, "design", "sekolorn") == "daburax":
+        return daburax_kernel_rates(a)
     from enterprise_inference_amd.ops import attention as A
     from enterprise_inference_amd.ops import latent_attention as LA
     from enterprise_inference_amd.ops import wkv as WK
@@ -554,4 +602,155 @@ def gapidra_kernel_rates(a) -> int:
         print(json.dumps(r_), flush=True)
     print(json.dumps({"metric": "design_kernel_rates", "design": "gapidra", "rows": rows}),
           flush=True)
+    return 0
+
+
+def daburax_kernel_rates(a) -> int:
+    """Achieved rates of the Daburax kernels beside their like kernels: the fixed-decay and the
+    gated linear scans beside the wkv scan at equal heads and head size (one 4096-token prompt:
+    tokens/s; a 64-row decode batch: state bytes/s); sink attention beside the paged flash
+    prefill and paged decode kernels of the Llama path at equal heads and lengths (prefill in
+    useful TFLOP/s, decode in cache bytes/s); the hyper-connection step over four streams beside
+    the fused add + RMS norm (bytes moved per second); the router.  One JSON line per kernel."""
+    import torch
+
+    from enterprise_inference_amd.ops import attention as A
+    from enterprise_inference_amd.ops import linear_scan as LS
+    from enterprise_inference_amd.ops import moe as M
+    from enterprise_inference_amd.ops import norm as N
+    from enterprise_inference_amd.ops import window_attention as WA
+    from enterprise_inference_amd.ops import wkv as WK
+    from enterprise_inference_amd.ops.rotary import rotary_frequencies
+
+    dev, bf = "cuda", torch.bfloat16
+    rows = []
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=dev)
+    # ---- scans: Hh heads of 64 x 64 (the wkv kernel's shape) and of 128 x 128
+    for Hh, D in ((32, 64), (16, 128)):
+        for (nseq, per) in ((1, 4096), (4, 2048), (64, 1)):
+            T = nseq * per
+            slots = torch.arange(nseq, dtype=torch.int32, device=dev)
+            cu = torch.arange(0, T + 1, per, dtype=torch.int32, device=dev)
+            pos = (torch.arange(T, dtype=torch.int32, device=dev) % per) + (5 if per == 1 else 0)
+            fused = (torch.randn(T, 4 * Hh * D + 2 * Hh, device=dev) * 0.3).to(bf)
+            inv, _ = rotary_frequencies(D, 1e6, None, dev)
+            for mode in ("decay", "exp_gates"):
+                spec = LS.ScanSpec(Hh, D, D, mode,
+                                   decay=torch.full((Hh,), 0.97, device=dev), cap=12.0,
+                                   inv_freq=inv if mode == "decay" else None,
+                                   rot_dims=D if mode == "decay" else 0, kscale=D ** -0.5,
+                                   gate_act="silu" if mode == "decay" else "sigmoid", eps=1e-5)
+                st = LS.ScanState.allocate(nseq, spec, dev)
+                t = _time(lambda: LS.linear_scan(fused, 0, Hh * D, 2 * Hh * D, 3 * Hh * D, spec,
+                                                 st, slots, cu, nseq, pos, None, None,
+                                                 4 * Hh * D, 4 * Hh * D + Hh))
+                rows.append({"kernel": f"linear_scan ({mode})", "heads": Hh, "dim": D,
+                             "seqs": nseq, "tokens_per_seq": per, "ms": t * 1e3,
+                             "tokens_per_s": T / t,
+                             "state_GBps": nseq * Hh * D * D * 4 * 2 / t / 1e9})
+            if D == 64:
+                HD, W = Hh * D, 2048
+                r, k, v, g = (torch.randn(T, HD, device=dev).to(bf) * 0.3 for _ in range(4))
+                dec = torch.randn(T, HD, device=dev) * 0.3
+                w0 = torch.full((HD,), -1.0, device=dev).to(bf)
+                u = (torch.randn(HD, device=dev) * 0.3).to(bf)
+                nw = torch.ones(HD, device=dev).to(bf)
+                S = torch.zeros(nseq, Hh, D, D, device=dev)
+                prev = torch.zeros(nseq, W, device=dev)
+                x = torch.randn(T, W, device=dev)
+                t = _time(lambda: WK.wkv_scan(r, k, v, g, dec, w0, u, nw, S, prev, x, slots, cu,
+                                              nseq, pos, None, 1e-5, Hh))
+                rows.append({"kernel": "wkv_scan", "heads": Hh, "dim": D, "seqs": nseq,
+                             "tokens_per_seq": per, "ms": t * 1e3, "tokens_per_s": T / t,
+                             "state_GBps": nseq * Hh * D * D * 4 * 2 / t / 1e9})
+    # ---- sink attention beside the paged kernels
+    bs, T = 128, 4096
+    pairs = T * (T + 1) // 2
+    B, L = 64, 4096
+    nb, nbd = T // bs, B * L // bs
+    pos = torch.arange(T, dtype=torch.int32, device=dev)
+    bt = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+    md = A.AttentionMetadata(
+        num_decode=0, num_prefill_tokens=T, slot_mapping=pos, positions=pos,
+        prefill_block_tables=bt, prefill_seq_lens=i32([T]), prefill_cu_q=i32([0, T]),
+        prefill_q_lens=[T])
+    btd = torch.arange(nbd, dtype=torch.int32, device=dev).view(B, L // bs)
+    posd = torch.full((B,), L - 1, dtype=torch.int32, device=dev)
+    mdd = A.AttentionMetadata(num_decode=B, num_prefill_tokens=0, slot_mapping=posd,
+                              positions=posd, decode_block_tables=btd,
+                              decode_seq_lens=i32([L] * B))
+    for H, G in ((8, 2), (16, 4)):
+        D = Dv = 128
+        spec = WA.WindowSpec(H, G, 1, D, Dv, 0, 0, mult=torch.full((H,), D ** -0.5, device=dev),
+                             sink=torch.zeros(H, device=dev))
+        kc = torch.randn(nb, bs, G * D, device=dev).to(bf)
+        vc = torch.randn(nb, G * Dv, bs, device=dev).to(bf)
+        q = torch.randn(T, H * D, device=dev).to(bf)
+        t = _time(lambda: WA.window_attention(q, kc, vc, md, spec, None))
+        rows.append({"kernel": "window_attn prefill (causal, sink)", "heads": H, "kv_heads": G,
+                     "dim": D, "vdim": Dv, "tokens": T, "ms": t * 1e3,
+                     "mfma": WA.mfma_ok(spec, bf, bs),
+                     "tflops": 2.0 * (D + Dv) * H * pairs / t / 1e12})
+        kcd = torch.randn(nbd, bs, G * D, device=dev).to(bf)
+        vcd = torch.randn(nbd, G * Dv, bs, device=dev).to(bf)
+        qd = q[:B].contiguous()
+        t = _time(lambda: WA.window_attention(qd, kcd, vcd, mdd, spec, None))
+        rows.append({"kernel": "window_attn decode (causal, sink)", "heads": H, "kv_heads": G,
+                     "batch": B, "context": L, "ms": t * 1e3,
+                     "cache_GBps": B * L * G * (D + Dv) * 2 / t / 1e9})
+        del kcd, vcd
+        kc = torch.randn(nb, G, bs, D, device=dev).to(bf)
+        vc = torch.randn(nb, G, D, bs, device=dev).to(bf)
+        q3 = torch.randn(T, H, D, device=dev).to(bf) * 0.1
+        qb2 = A.prefill_query_block(H, G, D, block_size=bs)
+        w2 = A.build_prefill_work([T], qb2)
+        wt = i32(w2)
+        t = _time(lambda: A.paged_prefill(q3, kc, vc, bt, i32([T]), i32([0, T]), wt, len(w2) // 2,
+                                          0.1))
+        rows.append({"kernel": "paged_prefill (flash)", "heads": H, "kv_heads": G,
+                     "head_dim": D, "tokens": T, "ms": t * 1e3,
+                     "tflops": 2.0 * 2 * D * H * pairs / t / 1e12})
+        kcd = torch.randn(nbd, G, bs, D, device=dev).to(bf)
+        vcd = torch.randn(nbd, G, D, bs, device=dev).to(bf)
+        lens = i32([L] * B)
+        qd3 = q3[:B].contiguous()
+        t = _time(lambda: A.paged_decode(qd3, kcd, vcd, btd, lens, 0.1))
+        rows.append({"kernel": "paged_decode", "heads": H, "kv_heads": G, "batch": B,
+                     "context": L, "ms": t * 1e3,
+                     "cache_GBps": B * L * G * D * 2 * 2 / t / 1e9})
+        del kcd, vcd
+    # ---- sublayer boundary over four streams beside the fused add + RMS norm
+    for W in (2048, 4096):
+        Tn, NS = 8192, 4
+        X = torch.randn(Tn, NS, W, device=dev)
+        y = torch.randn(Tn, W, device=dev).to(bf)
+        w1 = torch.zeros(W, device=dev).to(bf)
+        mix = torch.eye(NS, device=dev)
+        ones = torch.ones(NS, device=dev)
+        t = _time(lambda: N.hyper_step(X, 1e-5, y, mix, ones, 0.5, ones, w1, 1.0))
+        rows.append({"kernel": "hyper_step (4 streams)", "width": W, "rows": Tn, "ms": t * 1e3,
+                     "GBps": Tn * W * (2 * 4 * NS + 2 + 2) / t / 1e9})
+        res = torch.randn(Tn, W, device=dev).to(bf)
+        t = _time(lambda: N.fused_add_rms_norm(y, res, w1, 1e-5))
+        rows.append({"kernel": "fused_add_rms_norm", "width": W, "rows": Tn, "ms": t * 1e3,
+                     "GBps": Tn * W * (2 + 2 + 2 + 2) / t / 1e9})
+    # ---- router: softmax, correction, groups by their best member, identity outputs, gate
+    for E, W in ((10, 1024), (18, 2048)):
+        Tn = 8192
+        x = torch.randn(Tn, W, device=dev).to(bf)
+        wr = (torch.randn(E, W, device=dev) * 0.05).to(bf)
+        wsg = (torch.randn(W, device=dev) * 0.05).to(bf)
+        corr = torch.zeros(E, device=dev)
+        t = _time(lambda: M.route_grouped(x, wr, 2, 2, 1, 1.0, scoring="softmax",
+                                          group_score="max", correction=corr, identity=2,
+                                          gate_w=wsg))
+        rows.append({"kernel": "route_grouped (softmax, correction, identity, gate)",
+                     "outputs": E, "width": W, "rows": Tn, "ms": t * 1e3,
+                     "GBps": Tn * W * 2 / t / 1e9})
+        t = _time(lambda: M.route_grouped(x, wr, 2, 2, 1, 1.0))
+        rows.append({"kernel": "route_grouped (sigmoid)", "outputs": E, "width": W, "rows": Tn,
+                     "ms": t * 1e3, "GBps": Tn * W * 2 / t / 1e9})
+    for r_ in rows:
+        print(json.dumps(r_), flush=True)
+    print(json.dumps({"metric": "design_kernel_rates", "rows": rows}), flush=True)
     return 0

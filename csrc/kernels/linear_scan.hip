@@ -6,7 +6,8 @@
 // mode 0 (fixed decay, "retention"):  a_t = decay[h], b_t = 1.
 // mode 1 (exponential gates with a running maximum, "matrix memory"): per head two gate
 //   pre-activations x_i, x_f ride in the token's row;
-//     i = cap tanh(x_i / cap),  f = logsigmoid(cap tanh(x_f / cap)),  m_t = max(f + m_(t-1), i),
+//     i = cap tanh(x_i / cap),  f = logsigmoid(cap tanh(x_f / cap))   (cap 0: no cap),
+//     m_t = max(f + m_(t-1), i),
 //     a_t = exp(f + m_(t-1) - m_t),  b_t = exp(i - m_t),  n_t = a_t n_(t-1) + b_t k_t,
 //     o_t <- o_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6);       m starts at 0, S and n at zero.
 // Both: q and k may be rotated by the token's position on their first rot_dims entries (pairs
@@ -133,8 +134,8 @@ linear_scan_kernel(ScanArgs a) {
       if (threadIdx.x < nt) {                          // log gates of the chunk's tokens
         const T* xr = X + (long)(base + threadIdx.x) * a.ld;
         const float xi = ld_f32<T>(xr, a.i_off + h), xf = ld_f32<T>(xr, a.f_off + h);
-        gi[threadIdx.x] = a.cap * tanhf(xi / a.cap);
-        gf[threadIdx.x] = ls_logsigmoid(a.cap * tanhf(xf / a.cap));
+        gi[threadIdx.x] = a.cap > 0.f ? a.cap * tanhf(xi / a.cap) : xi;
+        gf[threadIdx.x] = ls_logsigmoid(a.cap > 0.f ? a.cap * tanhf(xf / a.cap) : xf);
       }
       __syncthreads();
       if (threadIdx.x == 0) {                          // the running maximum, token by token
@@ -232,7 +233,7 @@ EIA_API int eia_linear_scan(const void* x, long ld, int q_off, int k_off, int v_
                             const int* seq_lens, void* y, long ldy, float eps, int nseq, int H,
                             int D, int Dv, int mode, int gate_act, int is_bf16, hipStream_t st) {
   if (nseq < 0 || H < 1 || D < 1 || Dv < 1 || !x || !y || !S || !slots || !positions ||
-      (mode != 0 && mode != 1) || (mode == 0 && !decay) || (mode == 1 && (!N || !M || cap <= 0.f)) ||
+      (mode != 0 && mode != 1) || (mode == 0 && !decay) || (mode == 1 && (!N || !M || cap < 0.f)) ||
       rot_dims < 0 || rot_dims > D || (rot_dims & 1) || (rot_dims && !inv_freq) ||
       (gate_act != 0 && gate_act != 1))
     return EIA_BAD_SHAPE;

@@ -84,14 +84,17 @@ class DaburaxLayer(nn.Module):
         self.kind = spec["type"]
         if self.kind == "retention":
             rot = m.get("rot") or {}
+            # (a rot entry without dims rotates the whole head)
             self.mix = RetentionMixer(width, m["heads"], m["dim"], m.get("vdim", m["dim"]),
-                                      m["decay"], int(rot.get("dims", 0)),
+                                      m["decay"], int(rot.get("dims", m["dim"] if rot else 0)),
                                       float(rot.get("base", 10000.0)), rot.get("scaling"), eps,
                                       dtype, device)
         elif self.kind == "parallel":
             left, right = dict(m["left"]), dict(m["right"])
             left.setdefault("kv_heads", left["heads"])
             left.setdefault("vdim", left["dim"])
+            left.setdefault("scale", float(left["dim"]) ** -0.5)
+            right.setdefault("gate_cap", 0.0)           # (no cap)
             right.setdefault("vdim", right["dim"])
             self.mix = ParallelMixer(width, left, right, float(m.get("left_scale", 1.0)),
                                      float(m.get("right_scale", 1.0)), eps, dtype, device)

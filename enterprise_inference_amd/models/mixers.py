@@ -621,7 +621,7 @@ class RetentionMixer(_ScanMixerBase):
 class MatrixMemoryMixer(_ScanMixerBase):
     """Gated matrix memory: q = W_q x * dim^(-1/2), k [heads, dim], v [heads, vdim]; per head a
     log input gate i = cap tanh((W_i x + b_i) / cap) and a log forget gate f = logsigmoid(cap
-    tanh((W_f x + b_f) / cap)); with a running maximum m_t = max(f + m_(t-1), i) (from 0):
+    tanh((W_f x + b_f) / cap)) (``gate_cap`` 0: no cap); with a running maximum m_t = max(f + m_(t-1), i) (from 0):
     S_t = exp(f + m_(t-1) - m_t) S_(t-1) + exp(i - m_t) k v^T, n_t likewise with k alone,
     o = S_t^T q / (max(|n_t . q|, exp(-m_t)) + 1e-6).  Every head's o is divided by its root mean
     square; the concatenated heads are multiplied by the weight ``norm``, sigmoid(W_g x) and
@@ -667,7 +667,8 @@ class ParallelMixer(nn.Module):
         rot = left.get("rot") or {}
         self.left = SinkAttentionMixer(
             width, left["heads"], left["kv_heads"], left["dim"], left["vdim"], left["scale"],
-            int(rot.get("dims", 0)), float(rot.get("base", 10000.0)), rot.get("scaling"), eps,
+            int(rot.get("dims", left["dim"] if rot else 0)), float(rot.get("base", 10000.0)),
+            rot.get("scaling"), eps,
             dtype, device, window=int((left.get("mask") or {}).get("size", 0)),
             out_scale=left_scale, proj=self.proj, prefix="left.")
         self.right = MatrixMemoryMixer(width, right["heads"], right["dim"], right["vdim"],

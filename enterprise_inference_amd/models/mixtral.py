@@ -329,9 +329,13 @@ class GroupLimitedMoE(nn.Module):
         self.w2.weight_loader = lambda p, t, sid=None: p.data[sid].copy_(t)
         self.I = inter
         self.shared = LlamaMLP(hidden, shared_inter, act, dtype, device) if shared_inter else None
+        # zero until a checkpoint (or the random init) fills it: an all-zero row means the
+        # checkpoint has no gate, and the shared expert then counts whole
         self.shared_gate = None
+        self.gated = False
         if self.shared is not None and shared_gate:
             self.shared_gate = _param((hidden,), dtype, device)
+            self.shared_gate.data.zero_()
             self.shared_gate.weight_loader = lambda p, t, sid=None: p.data.copy_(t.reshape(-1))
 
     def _load_w13(self, param, loaded, shard_id):
@@ -341,6 +345,7 @@ class GroupLimitedMoE(nn.Module):
 
     def refresh(self) -> None:
         self.corr_f32.copy_(self.correction.float())
+        self.gated = self.shared_gate is not None and bool((self.shared_gate != 0).any())
 
     def forward(self, x: torch.Tensor, md=None) -> torch.Tensor:
         row_len = None
@@ -349,7 +354,8 @@ class GroupLimitedMoE(nn.Module):
         r = moe_ops.route_grouped(x, self.router, self.k, self.groups, self.keep,
                                   self.route_scale, row_len, scoring=self.scoring,
                                   group_score=self.group_score, correction=self.corr_f32,
-                                  identity=self.identity, gate_w=self.shared_gate)
+                                  identity=self.identity,
+                                  gate_w=self.shared_gate if self.gated else None)
         tw, ids = r[0], r[1]
         ident_w, sgate = (r[2], r[3]) if len(r) == 4 else (None, None)
         routed = moe_ops.fused_moe(x, self.w13, self.w2, tw, ids, (0, self.E), act=self.act)

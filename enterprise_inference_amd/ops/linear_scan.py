@@ -9,7 +9,7 @@ outer product to; the token's output reads the updated state:
 * ``mode="decay"`` (retention): a_t = decay[h], b_t = 1.
 * ``mode="exp_gates"`` (matrix memory with exponential gating): per head two gate
   pre-activations x_i, x_f per token; i = cap tanh(x_i / cap), f = logsigmoid(cap tanh(x_f /
-  cap)); a running maximum m_t = max(f + m_(t-1), i) (m starts at 0) keeps the exponentials
+  cap)) (cap 0: i = x_i, f = logsigmoid(x_f)); a running maximum m_t = max(f + m_(t-1), i) (m starts at 0) keeps the exponentials
   bounded: a_t = exp(f + m_(t-1) - m_t), b_t = exp(i - m_t); a normaliser n_t = a_t n_(t-1) +
   b_t k_t divides the output, o_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6).
 
@@ -129,9 +129,10 @@ def linear_scan(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: 
         g = f[:, g_off:g_off + H * Dv]
         y = torch.zeros(T, H, Dv)
         if exp_gates:
-            gi = spec.cap * torch.tanh(f[:, i_off:i_off + H] / spec.cap)
-            gf = torch.nn.functional.logsigmoid(spec.cap * torch.tanh(f[:, f_off:f_off + H]
-                                                                      / spec.cap))
+            soft = (lambda z: spec.cap * torch.tanh(z / spec.cap)) if spec.cap > 0 else \
+                (lambda z: z)
+            gi = soft(f[:, i_off:i_off + H])
+            gf = torch.nn.functional.logsigmoid(soft(f[:, f_off:f_off + H]))
         for s, (lo, hi) in enumerate(_seq_bounds(cu, nseq)):
             sl = int(slots[s])
             if hi <= lo or sl < 0:
@@ -176,7 +177,7 @@ def linear_scan(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: 
     if exp_gates:
         require(max(i_off, f_off) + H <= fused.shape[1] and state.n is not None and
                 state.m is not None and state.n.is_contiguous() and state.m.is_contiguous() and
-                spec.cap > 0, "linear_scan: gates")
+                spec.cap >= 0, "linear_scan: gates")
     else:
         require(spec.decay is not None and spec.decay.dtype == torch.float32 and
                 spec.decay.is_cuda and spec.decay.numel() == H, "linear_scan: decay per head")
