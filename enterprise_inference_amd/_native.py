@@ -78,6 +78,8 @@ _SIGNATURES = {
     "eia_linear_scan": [P, L, I, I, I, I, I, I, P, P, I, I, F, F, F, F, P, P, P, P, IP, IP, IP, IP,
                         P, L, F, I, I, I, I, I, I, I, S],
     "eia_moe_finish": [P, L, P, L, P, P, L, P, P, L, I, I, I, S],
+    "eia_linear_scan_chunked": [P, L, I, I, I, I, I, I, P, P, I, I, F, F, F, F, P, P, P, P, IP, IP,
+                                IP, P, L, F, I, I, I, I, I, I, I, IP, IP, I, P, P, P, P, P, P, S],
     "eia_hyper_step": [P, I, I, P, L, P, I, P, P, P, F, P, P, F, P, L, F, I, I, S],
     "eia_bigram_embed": [IP, P, F, P, I, L, L, IP, IP, IP, I, IP, P, I, I, I, I, I, S],
     "eia_relu2": [P, P, L, I, S],

@@ -575,11 +575,19 @@ class _ScanMixerBase(nn.Module):
             fused = fused.materialize() if fused.part.is_cuda else \
                 fused.part.sum(0) + (fused.bias.float() if fused.bias is not None else 0.0)
         o = self.offsets
+        # prompt portions: the step's chunk list, built once per step and shared by its layers
+        plan = None
+        if fused.is_cuda and md.seq_cu is not None:
+            if "scan_chunks" not in md.work_cache:
+                lens = [1] * md.num_decode + list(md.prefill_q_lens or [])
+                md.work_cache["scan_chunks"] = scan_ops.chunk_plan(
+                    lens if len(lens) == md.num_seqs else None, fused.device)
+            plan = md.work_cache["scan_chunks"]
         return scan_ops.linear_scan(
             fused, o["q"][0], o["k"][0], o["v"][0], o["g"][0], self.spec, state, md.seq_slots,
             md.seq_cu, md.num_seqs, md.positions,
             md.decode_seq_lens if md.seq_cu is None else None, norm_w,
-            o["i"][0] if "i" in o else 0, o["f"][0] if "f" in o else 0, out)
+            o["i"][0] if "i" in o else 0, o["f"][0] if "f" in o else 0, out, plan)
 
     def forward(self, xb: torch.Tensor, md: AttentionMetadata, state):
         # may return gemm.SplitK: the layer's boundary step reduces it

@@ -21,6 +21,12 @@ A sequence whose first row of the step is position 0 starts from the initial sta
 slot held, so freed slots are reused without clearing.  Batch layout: sequence ``s`` owns rows
 ``[cu[s], cu[s+1])`` of the step (``cu`` None: row ``s``, a pure decode step); ``slots[s]`` is its
 state slot (< 0: padding row, skipped).
+
+Prompt portions run a chunk-parallel form on the GPU (``chunk_plan``): the step's rows are cut
+into chunks of 32 tokens, every chunk's own contribution to the state is formed in parallel, a
+short scan over a sequence's chunks yields the state before each chunk, and the outputs of all
+chunks are formed in parallel from that state and the chunk's own tokens.  The token-by-token
+kernel serves decode steps (also inside captured graphs) and heads wider than 128.
 """
 
 from __future__ import annotations
@@ -80,6 +86,37 @@ class ScanState:
         return 4 * per
 
 
+CHUNK = 32                 # tokens per chunk of the chunk-parallel form (linear_scan.hip LC)
+CHUNK_MAX_DIM = 128        # ... and its largest dk / dv
+CHUNK_MIN_ROWS = 48        # a sequence with at least this many rows in the step selects it
+
+
+class ChunkPlan:
+    """A step's rows cut into chunks for the chunk-parallel form: ``chunks`` int32 [n, 4]
+    (sequence, first row, tokens, 0), ``seq_first`` int32 [nseq + 1] (first chunk of every
+    sequence), both on the device; ``rows`` the step's row count."""
+
+    __slots__ = ("chunks", "seq_first", "n", "rows")
+
+    def __init__(self, chunks, seq_first, n, rows):
+        self.chunks, self.seq_first, self.n, self.rows = chunks, seq_first, n, rows
+
+
+def chunk_plan(host_lens, device) -> Optional["ChunkPlan"]:
+    """The chunk list of a step whose sequences own ``host_lens`` rows each (batch order), or
+    None when no sequence is long enough for the chunk-parallel form to pay."""
+    if not host_lens or max(host_lens) < CHUNK_MIN_ROWS:
+        return None
+    chunks, first, row = [], [0], 0
+    for s, n in enumerate(host_lens):
+        for lo in range(0, n, CHUNK):
+            chunks += [s, row + lo, min(CHUNK, n - lo), 0]
+        row += n
+        first.append(len(chunks) // 4)
+    return ChunkPlan(torch.tensor(chunks, dtype=torch.int32, device=device).view(-1, 4),
+                     torch.tensor(first, dtype=torch.int32, device=device), len(chunks) // 4, row)
+
+
 def _seq_bounds(cu: Optional[torch.Tensor], nseq: int):
     if cu is None:
         return [(s, s + 1) for s in range(nseq)]
@@ -108,12 +145,14 @@ def linear_scan(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: 
                 spec: ScanSpec, state: ScanState, slots: torch.Tensor,
                 cu: Optional[torch.Tensor], nseq: int, positions: torch.Tensor,
                 seq_lens: Optional[torch.Tensor] = None, norm_w: Optional[torch.Tensor] = None,
-                i_off: int = 0, f_off: int = 0, out: Optional[torch.Tensor] = None
-                ) -> torch.Tensor:
+                i_off: int = 0, f_off: int = 0, out: Optional[torch.Tensor] = None,
+                plan: Optional[ChunkPlan] = None) -> torch.Tensor:
     """fused [T, *]: rows of one fused projection holding q [H*dk], k [H*dk], v [H*dv], the gate
     [H*dv] (and, with exponential gates, the H input-gate and H forget-gate pre-activations) at
     the given column offsets -> y [T, H*dv] in fused's dtype (``out``: a view to write into).
-    ``norm_w`` [H*dv]: weight after the head RMS norm.  Updates the sequences' slots."""
+    ``norm_w`` [H*dv]: weight after the head RMS norm.  Updates the sequences' slots.
+    ``plan``: the step's ``chunk_plan`` -- the GPU then runs the chunk-parallel form (heads up to
+    128 wide, outside graph capture)."""
     T = fused.shape[0]
     H, D, Dv = spec.heads, spec.dim, spec.vdim
     exp_gates = spec.mode == "exp_gates"
@@ -190,6 +229,23 @@ def linear_scan(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: 
             (cu is None or cu.dtype == torch.int32), "linear_scan: int32 metadata")
     require(norm_w is None or (norm_w.dtype == fused.dtype and norm_w.is_contiguous() and
                                norm_w.numel() == H * Dv), "linear_scan: norm weight")
+    if (plan is not None and plan.n and max(D, Dv) <= CHUNK_MAX_DIM and cu is not None
+            and plan.rows == T and not torch.cuda.is_current_stream_capturing()):
+        dev = fused.device
+        f32 = lambda *shape: torch.empty(*shape, dtype=torch.float32, device=dev)
+        wsS, wsG = f32(plan.n, H, D, Dv), f32(plan.n, H)
+        wsN = f32(plan.n, H, D) if exp_gates else None
+        la, lb, nm = (f32(T, H), f32(T, H), f32(T, H)) if exp_gates else (None, None, None)
+        check(lib().eia_linear_scan_chunked(
+            ptr(fused), fused.stride(0), q_off, k_off, v_off, g_off, i_off, f_off,
+            ptr(spec.decay), ptr(spec.inv_freq), spec.rot_dims, 1 if spec.rot_half else 0,
+            float(spec.qscale), float(spec.kscale), float(spec.cap), float(spec.out_scale),
+            ptr(norm_w), ptr(state.S), ptr(state.n), ptr(state.m), ptr(slots), ptr(cu),
+            ptr(positions), ptr(out), out.stride(0), float(spec.eps), nseq, H, D, Dv,
+            1 if exp_gates else 0, 0 if spec.gate_act == "silu" else 1, 1 if bf else 0,
+            ptr(plan.chunks), ptr(plan.seq_first), plan.n, ptr(wsS), ptr(wsN), ptr(wsG), ptr(la),
+            ptr(lb), ptr(nm), stream(fused)), "linear_scan_chunked")
+        return out
     check(lib().eia_linear_scan(
         ptr(fused), fused.stride(0), q_off, k_off, v_off, g_off, i_off, f_off, ptr(spec.decay),
         ptr(spec.inv_freq), spec.rot_dims, 1 if spec.rot_half else 0, float(spec.qscale),

@@ -196,10 +196,12 @@ def _scan_offsets(H, D, Dv):
         2 * H * D + 2 * H * Dv + H
 
 
-def case_retention_scan(device, dtype, H=3, D=10, Dv=6, dims=4, half=True, T=75):
+def case_retention_scan(device, dtype, H=3, D=10, Dv=6, dims=4, half=True, T=75, chunked=False):
     """The fixed-decay recurrence alone: a sequence run whole, and run in portions (down to one
     token) beside another sequence on slots that held something else before; one early token is
-    made to stand out so that a slow head still shows it 70 tokens later."""
+    made to stand out so that a slow head still shows it 70 tokens later.  ``chunked``: long
+    portions take the chunk-parallel form (their chunk list is handed over), short ones the
+    token-by-token form, on the same slots."""
     from enterprise_inference_amd.ops import linear_scan as ls
     from enterprise_inference_amd.ops.rotary import rotary_frequencies
     g = torch.Generator().manual_seed(11)
@@ -235,8 +237,9 @@ def case_retention_scan(device, dtype, H=3, D=10, Dv=6, dims=4, half=True, T=75)
             other = fd[:2] * 0.5                       # a second sequence beside it, slot 0
             rows = torch.cat([other, fd[lo:hi]])
             pos = _i32([0, 1] + list(range(lo, hi)), device)
+            plan = ls.chunk_plan([2, hi - lo], device) if chunked else None
             y = ls.linear_scan(rows, qo, ko, vo, go, spec, state, _i32([0, sl], device),
-                               _i32([0, 2, 2 + hi - lo], device), 2, pos)
+                               _i32([0, 2, 2 + hi - lo], device), 2, pos, plan=plan)
             out.append(y[2:])
         return torch.cat(out)
 
@@ -246,13 +249,16 @@ def case_retention_scan(device, dtype, H=3, D=10, Dv=6, dims=4, half=True, T=75)
     cuts = [c for c in (0, 2, 3, 19, 20, 36, 37, 39, 70) if c < T] + [T]
     got = run([(2, a, b) for a, b in zip(cuts[:-1], cuts[1:])])
     assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
+    if chunked and T > 130:                            # long portions that start from a held state
+        got = run([(2, 0, 65), (2, 65, 66), (2, 66, T)])
+        assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
     # pure decode rows (no row ranges): slot 1 still holds the state after T tokens
     y = ls.linear_scan(fd[T - 1:T], qo, ko, vo, go, spec, state, _i32([1], device), None, 1,
                        _i32([T], device), _i32([T + 1], device))
     assert y.shape == (1, H * Dv) and bool(torch.isfinite(y.float()).all())
 
 
-def case_memory_scan(device, dtype, H=2, D=6, Dv=10, T=70, cap=8.0):
+def case_memory_scan(device, dtype, H=2, D=6, Dv=10, T=70, cap=8.0, chunked=False):
     """The gated matrix memory alone: whole against portions on stale slots; gate
     pre-activations large enough to reach the soft cap, so the running maximum moves and the
     normaliser's two branches (|n . q| and exp(-m)) are both taken."""
@@ -287,10 +293,11 @@ def case_memory_scan(device, dtype, H=2, D=6, Dv=10, T=70, cap=8.0):
     def run(slot, cuts):
         out = []
         for lo, hi in zip(cuts[:-1], cuts[1:]):
+            plan = ls.chunk_plan([hi - lo], device) if chunked else None
             out.append(ls.linear_scan(fd[lo:hi], qo, ko, vo, go, spec, state, _i32([slot], device),
                                       _i32([0, hi - lo], device), 1,
                                       _i32(list(range(lo, hi)), device), None, nw.to(device),
-                                      io, fo))
+                                      io, fo, plan=plan))
         return torch.cat(out)
 
     tk = ktol(dtype) * 4
@@ -298,6 +305,9 @@ def case_memory_scan(device, dtype, H=2, D=6, Dv=10, T=70, cap=8.0):
     assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
     got = run(1, [c for c in (0, 1, 3, 18, 19, 35, 52, 53) if c < T] + [T])
     assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
+    if chunked and T > 130:
+        got = run(0, [0, 65, 66, T])
+        assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
 
 
 def case_sink_needle(device, dtype, H=4, G=2, D=16, Dv=8, n=150, bs=16, size=0):

@@ -44,6 +44,23 @@ def test_memory_scan(shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(3, 10, 6, 4, True, 150), (2, 64, 48, 32, True, 140),
+                                   (2, 128, 128, 128, False, 135), (1, 24, 128, 0, True, 200)],
+                         ids=lambda s: "-".join(map(str, s)))
+def test_retention_scan_chunk_parallel(shape, dtype):
+    H, D, Dv, dims, half, T = shape
+    K.case_retention_scan("cuda", dtype, H, D, Dv, dims, half, T, chunked=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(2, 6, 10, 150), (3, 48, 64, 140), (2, 128, 72, 135),
+                                   (1, 128, 128, 200)], ids=lambda s: "-".join(map(str, s)))
+def test_memory_scan_chunk_parallel(shape, dtype):
+    H, D, Dv, T = shape
+    K.case_memory_scan("cuda", dtype, H, D, Dv, T, chunked=True)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("shape", [
     # H, G, D, Dv, window, tokens, page
     (4, 2, 16, 8, 0, 150, 16),
@@ -90,8 +107,8 @@ def test_generate_through_engine(dtype):
     K.case_generate("cuda", dtype, C.config_a)
 
 
-def test_generate_config_c_bf16():
-    K.case_generate("cuda", torch.bfloat16, C.config_c)
+def test_generate_graph_decode_config_c():
+    K.case_generate("cuda", torch.bfloat16, C.config_c, expect_graphs=True)
 
 
 def test_native_library_loaded():
