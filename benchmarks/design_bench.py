@@ -641,13 +641,17 @@ def daburax_kernel_rates(a) -> int:
                                    rot_dims=D if mode == "decay" else 0, kscale=D ** -0.5,
                                    gate_act="silu" if mode == "decay" else "sigmoid", eps=1e-5)
                 st = LS.ScanState.allocate(nseq, spec, dev)
-                t = _time(lambda: LS.linear_scan(fused, 0, Hh * D, 2 * Hh * D, 3 * Hh * D, spec,
-                                                 st, slots, cu, nseq, pos, None, None,
-                                                 4 * Hh * D, 4 * Hh * D + Hh))
-                rows.append({"kernel": f"linear_scan ({mode})", "heads": Hh, "dim": D,
-                             "seqs": nseq, "tokens_per_seq": per, "ms": t * 1e3,
-                             "tokens_per_s": T / t,
-                             "state_GBps": nseq * Hh * D * D * 4 * 2 / t / 1e9})
+                forms = [("token by token", None)]
+                if per > 1:
+                    forms.append(("chunk-parallel", LS.chunk_plan([per] * nseq, dev)))
+                for form, plan in forms:
+                    t = _time(lambda: LS.linear_scan(fused, 0, Hh * D, 2 * Hh * D, 3 * Hh * D,
+                                                     spec, st, slots, cu, nseq, pos, None, None,
+                                                     4 * Hh * D, 4 * Hh * D + Hh, plan=plan))
+                    rows.append({"kernel": f"linear_scan ({mode}, {form})", "heads": Hh, "dim": D,
+                                 "seqs": nseq, "tokens_per_seq": per, "ms": t * 1e3,
+                                 "tokens_per_s": T / t,
+                                 "state_GBps": nseq * Hh * D * D * 4 * 2 / t / 1e9})
             if D == 64:
                 HD, W = Hh * D, 2048
                 r, k, v, g = (torch.randn(T, HD, device=dev).to(bf) * 0.3 for _ in range(4))

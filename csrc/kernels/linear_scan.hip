@@ -279,6 +279,7 @@ EIA_API int eia_linear_scan(const void* x, long ld, int q_off, int k_off, int v_
 // beside the projections.
 constexpr int LC = 32;                      // tokens per chunk
 constexpr int LD = 128;                     // largest dk / dv of this form
+constexpr int LP = LD + 4;                  // LDS row pitch: 16-byte rows that rotate the banks
 
 struct ChunkArgs {
   const int* chunks;                        // [nchunk, 4]: sequence, first row, tokens, unused
@@ -334,7 +335,7 @@ ls_gates_kernel(ScanArgs a, ChunkArgs c) {
 // Stages rotated, scaled q or k rows ([LC][LD], zero beyond n tokens / D channels).
 template <typename T>
 EIA_DEV void ls_stage_rot(const ScanArgs& a, const T* X, int row0, int n, long off, float scale,
-                          float (*dst)[LD]) {
+                          float (*dst)[LP]) {
   const int hd = a.rot_dims >> 1;
   for (int idx = threadIdx.x; idx < LC * LD; idx += blockDim.x) {
     const int t = idx / LD, j = idx % LD;
@@ -385,7 +386,7 @@ EIA_DEV void ls_chunk_decay(const ScanArgs& a, const ChunkArgs& c, int row0, int
 template <typename T>
 __global__ void __launch_bounds__(256)
 ls_chunk_state_kernel(ScanArgs a, ChunkArgs c) {
-  __shared__ __align__(16) float sk[LC][LD], sv[LC][LD];
+  __shared__ __align__(16) float sk[LC][LP], sv[LC][LD];
   __shared__ float sA[LC], sB[LC];
   const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int s = c.chunks[4 * ch], row0 = c.chunks[4 * ch + 1], n = c.chunks[4 * ch + 2];
@@ -471,7 +472,7 @@ ls_chunk_scan_kernel(ScanArgs a, ChunkArgs c) {
 template <typename T>
 __global__ void __launch_bounds__(256)
 ls_chunk_out_kernel(ScanArgs a, ChunkArgs c) {
-  __shared__ __align__(16) float sq[LC][LD], sk[LC][LD], sv[LC][LD];
+  __shared__ __align__(16) float sq[LC][LP], sk[LC][LP], sv[LC][LD];
   __shared__ float P[LC][LC + 1];
   __shared__ float sA[LC], sB[LC], snq[LC], red[LC][2];
   const int ch = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;

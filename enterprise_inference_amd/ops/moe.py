@@ -186,7 +186,11 @@ def fused_moe(x: torch.Tensor, w13: torch.Tensor, w2: torch.Tensor, topk_w: torc
     if act == "silu" and avg <= 96 and _grouped_ok(x, w13, w2):
         return _fused_moe_grouped(x, w13, w2, topk_w, topk_ids, e_lo, e_hi,
                                   defer_combine=defer_combine)
-    if act == "silu" and _mfma_ok(x, w13, w2) and (avg <= MFMA_MAX_ROWS or capturable):
+    # (small experts stay on the grouped MFMA kernel at any row count: their per-expert library
+    # GEMMs are launch- and read-back-bound, not MFMA-bound)
+    if act == "silu" and _mfma_ok(x, w13, w2) and (
+            avg <= MFMA_MAX_ROWS or capturable
+            or (w13.shape[1] // 2) * H <= UNGATED_SMALL_EXPERT):
         return _fused_moe_grouped(x, w13, w2, topk_w, topk_ids, e_lo, e_hi, mfma=True)
     if capturable:
         if act == "silu" and _grouped_ok(x, w13, w2):
