@@ -234,7 +234,11 @@ def run(a) -> int:
                              "benchmarks/design_bench.py); run s or s6")
         if design == "daburax":
             z = DSIZES[name]
-            pair = (("Daburax", daburax_config(z)), ("Sekolorn", sekolorn_like(z)))
+            # (Sekolorn's engines at width 2048 are switched off, see GATED: the larger size
+            # runs beside the Mixtral-style decoder instead)
+            other = ("Sekolorn", sekolorn_like(z)) if name == "ds" else \
+                ("Mixtral-style", mixtral_config(z))
+            pair = (("Daburax", daburax_config(z)), other)
         elif design == "gapidra":
             z = dict(GSIZES[name], layers=6)
             pair = (("Gapidra", gapidra_config(z)), ("Mistral-style", mistral_config(z)))
@@ -645,6 +649,7 @@ def daburax_kernel_rates(a) -> int:
                 if per > 1:
                     forms.append(("chunk-parallel", LS.chunk_plan([per] * nseq, dev)))
                 for form, plan in forms:
+                    LS.FORCE_CHUNKED = plan is not None
                     t = _time(lambda: LS.linear_scan(fused, 0, Hh * D, 2 * Hh * D, 3 * Hh * D,
                                                      spec, st, slots, cu, nseq, pos, None, None,
                                                      4 * Hh * D, 4 * Hh * D + Hh, plan=plan))

@@ -33,6 +33,7 @@ from __future__ import annotations
 
 import dataclasses
 import math
+import os
 from typing import Optional
 
 import torch
@@ -89,6 +90,8 @@ class ScanState:
 CHUNK = 32                 # tokens per chunk of the chunk-parallel form (linear_scan.hip LC)
 CHUNK_MAX_DIM = 128        # ... and its largest dk / dv
 CHUNK_MIN_ROWS = 48        # a sequence with at least this many rows in the step selects it
+# tests and measurements: take the chunk-parallel form whenever a plan is handed over
+FORCE_CHUNKED = os.environ.get("EIA_SCAN_FORCE_CHUNKED", "0") == "1"
 
 
 class ChunkPlan:
@@ -96,10 +99,20 @@ class ChunkPlan:
     (sequence, first row, tokens, 0), ``seq_first`` int32 [nseq + 1] (first chunk of every
     sequence), both on the device; ``rows`` the step's row count."""
 
-    __slots__ = ("chunks", "seq_first", "n", "rows")
+    __slots__ = ("chunks", "seq_first", "n", "rows", "nseq", "longest")
 
-    def __init__(self, chunks, seq_first, n, rows):
+    def __init__(self, chunks, seq_first, n, rows, nseq=1, longest=0):
         self.chunks, self.seq_first, self.n, self.rows = chunks, seq_first, n, rows
+        self.nseq, self.longest = nseq, longest
+
+    def pays(self, heads: int, dim: int, cus: int = 256) -> bool:
+        """Whether the chunk-parallel form beats the token-by-token one for a layer of ``heads``
+        heads up to ``dim`` wide: the latter walks the longest sequence with one workgroup per
+        (sequence, head) at about 0.5 us a token (0.85 us above 64), the former costs about 5 ns
+        (7 ns) per token and head over all rows (MI355X, measured on 4096-token prompts)."""
+        wide = dim > 64
+        serial = self.longest * (0.85 if wide else 0.5) * -(-self.nseq * heads // cus)
+        return self.rows * heads * (0.0072 if wide else 0.0052) < serial
 
 
 def chunk_plan(host_lens, device) -> Optional["ChunkPlan"]:
@@ -114,7 +127,8 @@ def chunk_plan(host_lens, device) -> Optional["ChunkPlan"]:
         row += n
         first.append(len(chunks) // 4)
     return ChunkPlan(torch.tensor(chunks, dtype=torch.int32, device=device).view(-1, 4),
-                     torch.tensor(first, dtype=torch.int32, device=device), len(chunks) // 4, row)
+                     torch.tensor(first, dtype=torch.int32, device=device), len(chunks) // 4, row,
+                     len(host_lens), max(host_lens))
 
 
 def _seq_bounds(cu: Optional[torch.Tensor], nseq: int):
@@ -230,7 +244,8 @@ def linear_scan(fused: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: 
     require(norm_w is None or (norm_w.dtype == fused.dtype and norm_w.is_contiguous() and
                                norm_w.numel() == H * Dv), "linear_scan: norm weight")
     if (plan is not None and plan.n and max(D, Dv) <= CHUNK_MAX_DIM and cu is not None
-            and plan.rows == T and not torch.cuda.is_current_stream_capturing()):
+            and plan.rows == T and (FORCE_CHUNKED or plan.pays(H, max(D, Dv)))
+            and not torch.cuda.is_current_stream_capturing()):
         dev = fused.device
         f32 = lambda *shape: torch.empty(*shape, dtype=torch.float32, device=dev)
         wsS, wsG = f32(plan.n, H, D, Dv), f32(plan.n, H)

@@ -183,6 +183,12 @@ def case_route(device, dtype):
             assert iw is None
 
 
+def _force_chunked(on):
+    """Tests that hand a chunk list over want the chunk-parallel form whatever the cost rule says."""
+    from enterprise_inference_amd.ops import linear_scan as ls
+    ls.FORCE_CHUNKED = bool(on)
+
+
 def _scan_inputs(g, T, H, D, Dv, dtype, gates):
     width = 2 * H * D + 2 * H * Dv + (2 * H if gates else 0) + 3
     fused = torch.randn(T, width, generator=g)
@@ -229,6 +235,7 @@ def case_retention_scan(device, dtype, H=3, D=10, Dv=6, dims=4, half=True, T=75,
     state = ls.ScanState.allocate(3, spec, device)
     state.S.fill_(5.0)                                 # stale slots
     fd = fused.to(device)
+    _force_chunked(chunked)
 
     def run(chunks):
         """chunks: (slot, lo, hi) of the one sequence, each as its own step."""
@@ -252,6 +259,7 @@ def case_retention_scan(device, dtype, H=3, D=10, Dv=6, dims=4, half=True, T=75,
     if chunked and T > 130:                            # long portions that start from a held state
         got = run([(2, 0, 65), (2, 65, 66), (2, 66, T)])
         assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
+    _force_chunked(False)
     # pure decode rows (no row ranges): slot 1 still holds the state after T tokens
     y = ls.linear_scan(fd[T - 1:T], qo, ko, vo, go, spec, state, _i32([1], device), None, 1,
                        _i32([T], device), _i32([T + 1], device))
@@ -289,6 +297,7 @@ def case_memory_scan(device, dtype, H=2, D=6, Dv=10, T=70, cap=8.0, chunked=Fals
     state.n.fill_(-2.0)
     state.m.fill_(4.0)
     fd = fused.to(device)
+    _force_chunked(chunked)
 
     def run(slot, cuts):
         out = []
@@ -308,6 +317,7 @@ def case_memory_scan(device, dtype, H=2, D=6, Dv=10, T=70, cap=8.0, chunked=Fals
     if chunked and T > 130:
         got = run(0, [0, 65, 66, T])
         assert np.allclose(_np(got), want, atol=tk, rtol=tk), np.abs(_np(got) - want).max()
+    _force_chunked(False)
 
 
 def case_sink_needle(device, dtype, H=4, G=2, D=16, Dv=8, n=150, bs=16, size=0):
