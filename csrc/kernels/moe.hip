@@ -538,7 +538,10 @@ EIA_API int eia_moe_combine_sk(const float* part, int sk, int rows, const float*
 // row [H]; sgate[t] = sigmoid(wsg . x), a token's gate for an always-on expert.
 // One wave per token: lanes split the width for the dot products; up to 64 outputs the lanes then
 // rank themselves with shuffles (lane e = output e), above that lane 0 selects serially (E <= 256).
-template <typename T>
+// SPLIT (small batches): one workgroup per token, its four waves share the dot products (wave w
+// takes the 8-output passes w, w + 4, ...; the last wave also the gate row) and wave 0 ranks --
+// a lone wave's chain of dependent weight loads is what a decode step would otherwise wait for.
+template <typename T, bool SPLIT>
 __global__ void __launch_bounds__(256)
 route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr, int H, int T_,
                      int E, int k, int ngroups, int keep, float route_scale,
@@ -552,26 +555,30 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
   __shared__ float sc[4][256];
   __shared__ float ch[4][256];
   __shared__ unsigned char ok[4][256];
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + wave;
+  const int wid = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int wave = SPLIT ? 0 : wid;            // (row of the LDS arrays)
+  const int t = SPLIT ? (int)blockIdx.x : (int)blockIdx.x * 4 + wid;
   if (t >= T_) return;
   const T* xr = x + (long)t * ldx;
   float mine = -INFINITY;                      // lane e keeps output e's logit (E <= 64)
   const bool vec8 = (H & 7) == 0 && (ldx & 7) == 0;
-  for (int e0 = 0; e0 < E; e0 += 8) {          // eight outputs per pass over the token's row
+  // eight outputs per pass over the token's row
+  for (int e0 = SPLIT ? 8 * wid : 0; e0 < E; e0 += SPLIT ? 32 : 8) {
     float p[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     if constexpr (sizeof(T) == 2) {
       if (vec8) {                              // 16-byte loads: 8 consecutive channels per lane
         for (int c = lane * 8; c < H; c += 512) {
+          // all nine loads are issued before the first use (outputs past E re-read the last
+          // row: no branch between the loads)
           const bf16x8 xv = *reinterpret_cast<const bf16x8*>(xr + c);
+          bf16x8 wv[8];
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            if (e0 + j < E) {
-              const bf16x8 wv = *reinterpret_cast<const bf16x8*>(wr + (long)(e0 + j) * H + c);
+          for (int j = 0; j < 8; ++j)
+            wv[j] = *reinterpret_cast<const bf16x8*>(wr + (long)min(e0 + j, E - 1) * H + c);
 #pragma unroll
-              for (int q = 0; q < 8; ++q) p[j] += bf2f(xv[q]) * bf2f(wv[q]);
-            }
-          }
+          for (int j = 0; j < 8; ++j)
+#pragma unroll
+            for (int q = 0; q < 8; ++q) p[j] += bf2f(xv[q]) * bf2f(wv[j][q]);
         }
       }
     }
@@ -592,11 +599,17 @@ route_grouped_kernel(const T* __restrict__ x, long ldx, const T* __restrict__ wr
       }
     }
   }
-  if (wsg) {
+  if (wsg && (!SPLIT || wid == 3)) {
     float p = 0.f;
+#pragma unroll 4
     for (int c = lane; c < H; c += 64) p += ld_f32<T>(xr, c) * ld_f32<T>(wsg, c);
     p = wave_sum(p);
     if (lane == 0) sgate[t] = 1.0f / (1.0f + expf(-p));
+  }
+  if constexpr (SPLIT) {
+    __syncthreads();                           // every wave's logits are in sc[0]
+    if (wid != 0) return;
+    mine = lane < E ? sc[0][lane] : -INFINITY;
   }
   const bool pad = row_len && row_len[t] == 0;
   const int per = E / ngroups;
@@ -724,15 +737,18 @@ EIA_API int eia_moe_route_grouped(const void* x, long ldx, const void* wr, int H
       (gmode != 0 && gmode != 1) || n_real < 0 || n_real > E || (wsg && !sgate))
     return EIA_BAD_SHAPE;
   if (T <= 0) return EIA_OK;
-  dim3 grid((T + 3) / 4), block(256);
-  if (is_bf16)
-    hipLaunchKernelGGL((route_grouped_kernel<bf16_t>), grid, block, 0, st, (const bf16_t*)x, ldx,
-                       (const bf16_t*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,
-                       extra, scoring, gmode, corr, n_real, ident_w, (const bf16_t*)wsg, sgate);
-  else
-    hipLaunchKernelGGL((route_grouped_kernel<float>), grid, block, 0, st, (const float*)x, ldx,
-                       (const float*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,
-                       extra, scoring, gmode, corr, n_real, ident_w, (const float*)wsg, sgate);
+  const bool split = T <= 512;                 // fewer tokens than two workgroups per CU
+  dim3 grid(split ? T : (T + 3) / 4), block(256);
+#define RG_LAUNCH(TT, SP)                                                                        \
+  hipLaunchKernelGGL((route_grouped_kernel<TT, SP>), grid, block, 0, st, (const TT*)x, ldx,      \
+                     (const TT*)wr, H, T, E, k, ngroups, keep, route_scale, tw, ids, row_len,    \
+                     extra, scoring, gmode, corr, n_real, ident_w, (const TT*)wsg, sgate)
+  if (is_bf16) {
+    if (split) RG_LAUNCH(bf16_t, true); else RG_LAUNCH(bf16_t, false);
+  } else {
+    if (split) RG_LAUNCH(float, true); else RG_LAUNCH(float, false);
+  }
+#undef RG_LAUNCH
   EIA_LAUNCH_CHECK();
 }
 
