@@ -341,6 +341,7 @@ class DaburaxForCausalLM(nn.Module):
                 mix = self.get_submodule(name.rsplit(".", 1)[0])
                 if isinstance(mix, ParallelMixer):
                     p.data[:, mix.lw:mix.lw_pad].zero_()
+                    p.data[:, mix.lw_pad + mix.rw:].zero_()
             else:
                 p.data.copy_(rnd(p.shape[-1] ** -0.5))
 

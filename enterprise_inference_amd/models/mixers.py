@@ -685,9 +685,10 @@ class ParallelMixer(nn.Module):
         self.lw = left["heads"] * left["vdim"]
         self.rw = right["heads"] * right["vdim"]
         self.lw_pad = -(-self.lw // 8) * 8           # the right heads start 16-byte aligned
-        # output projection over [left heads | pad | right heads]; the checkpoint's two output
-        # matrices load into its column ranges
-        self.o = _param((width, self.lw_pad + self.rw), dtype, device)
+        self.row = -(-(self.lw_pad + self.rw) // 8) * 8     # ... and so does every row
+        # output projection over [left heads | pad | right heads | pad]; the checkpoint's two
+        # output matrices load into its column ranges (pad columns stay zero)
+        self.o = _param((width, self.row), dtype, device)
         self.o.data.zero_()
         self.o.weight_loader = self._load_o
 
@@ -706,10 +707,12 @@ class ParallelMixer(nn.Module):
         kv, state = cache
         fused = self.proj(xb)
         T = xb.shape[0]
-        heads = torch.empty(T, self.lw_pad + self.rw, dtype=xb.dtype, device=xb.device)
+        heads = torch.empty(T, self.row, dtype=xb.dtype, device=xb.device)
         if self.lw_pad != self.lw:
             heads[:, self.lw:self.lw_pad].zero_()
+        if self.row != self.lw_pad + self.rw:
+            heads[:, self.lw_pad + self.rw:].zero_()
         self.left.attend(fused, md, kv, out=heads[:, :self.lw])
-        self.right.attend(fused, md, state, out=heads[:, self.lw_pad:])
+        self.right.attend(fused, md, state, out=heads[:, self.lw_pad:self.lw_pad + self.rw])
         # may return gemm.SplitK: the layer's boundary step reduces it
         return gemm.linear(heads, self.o, defer_reduce=True)

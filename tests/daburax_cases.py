@@ -365,6 +365,52 @@ def case_sink_needle(device, dtype, H=4, G=2, D=16, Dv=8, n=150, bs=16, size=0):
                 assert d < (2e-4 if dtype == torch.float32 else 4e-2), (j, p, a, d)
 
 
+def case_expert_block(device, dtype, W=46, ff=20, E=6, ident=2, top=3, cnt=4, keep=2, shared=12,
+                      T=21):
+    """The whole expert block (router, gated experts, identity outputs, gated shared expert,
+    final sum) against the plain rule, at sizes that take the per-expert, the grouped
+    weight-streaming and the grouped matrix-core forms; corrections 1.5 apart so that no choice
+    rests on a close call."""
+    from enterprise_inference_amd.models.mixtral import GroupLimitedMoE
+    g = torch.Generator().manual_seed(17)
+    mlp = {"expert": {"ff": ff}, "router": {"experts": E, "identity": ident, "top": top,
+                                            "groups": {"count": cnt, "keep": keep}}}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    Wt = {}
+    mat = lambda n, k, s=1.0: (torch.randn(n, k, generator=g) * (s / k ** 0.5)).to(dtype).float()
+    Wt["router"] = mat(E + ident, W, 1.5)
+    Wt["correction"] = (torch.randperm(E + ident, generator=g).float() * 1.5).to(dtype).float()
+    for e in range(E):
+        Wt[f"e{e}.gate"], Wt[f"e{e}.up"], Wt[f"e{e}.down"] = mat(ff, W, 1.5), mat(ff, W, 1.5), \
+            mat(W, ff, 0.7)
+    if shared:
+        Wt["shared.gate"], Wt["shared.up"] = mat(shared, W, 1.5), mat(shared, W, 1.5)
+        Wt["shared.down"], Wt["shared.sg"] = mat(W, shared, 0.7), mat(1, W, 2.0)
+    mod = GroupLimitedMoE(W, ff, E, top, cnt, keep, ident, shared, dtype=dtype,
+                          device=torch.device(device))
+    with torch.no_grad():
+        mod.router.copy_(Wt["router"])
+        mod.correction.copy_(Wt["correction"])
+        for e in range(E):
+            mod.w13[e, :ff].copy_(Wt[f"e{e}.gate"])
+            mod.w13[e, ff:].copy_(Wt[f"e{e}.up"])
+            mod.w2[e].copy_(Wt[f"e{e}.down"])
+        if shared:
+            mod.shared.gate_up_proj.weight[:shared].copy_(Wt["shared.gate"])
+            mod.shared.gate_up_proj.weight[shared:].copy_(Wt["shared.up"])
+            mod.shared.down_proj.weight.copy_(Wt["shared.down"])
+            mod.shared_gate.copy_(Wt["shared.sg"].reshape(-1))
+    mod.refresh()
+    x = torch.randn(T, W, generator=g).to(dtype)
+    with torch.no_grad():
+        got = mod(x.to(device))
+    W64 = {k: _np(v) for k, v in Wt.items()}
+    want = np.stack([O.moe(_np(x[t]), W64, "", mlp) for t in range(T)])
+    err = np.abs(_np(got) - want).max() / np.abs(want).max()
+    assert err < (1e-4 if dtype == torch.float32 else 3e-2), (W, ff, T, err)
+
+
 def case_frequencies():
     """Position interpolation with a lone factor divides every frequency."""
     from enterprise_inference_amd.ops.rotary import rotary_frequencies

@@ -93,6 +93,18 @@ def config_c():
                                rd=32, rv=32, cap=12.0, ls=0.7, rs=1.4), experts=0)]}
 
 
+def config_d():
+    """One learned stream; an attention side whose sizes take the matrix-core form beside a
+    recurrent side of odd width (3 heads of 5), so the shared row of the two needs padding; a
+    retention layer whose rotation covers part of a 24-wide head."""
+    return {"architecture": "Daburax", "vocab": 80, "width": 64, "norm": {"eps": 1e-5},
+            "residual_mult": 1.5, "streams": 1, "embedding": {"scale": 0.5},
+            "layers": [moe(par(lh=2, lg=1, ld=16, lv=16, ldims=8, lbase=300.0, factor=3.0,
+                               lscale=0.25, rh=3, rd=8, rv=5, cap=6.0, ls=0.9, rs=1.1),
+                           experts=4, top=2, identity=0, count=2, keep=2, ff=16, shared=16),
+                       moe(ret(heads=2, dim=24, vdim=16, decay=(0.9, 0.99), dims=10), experts=0)]}
+
+
 def random_weights(cfg: dict, seed: int = 0, dtype=torch.float32, decisive: bool = False,
                    tie_qk: bool = False) -> dict:
     """A checkpoint for ``cfg`` under the design's tensor names (values rounded to ``dtype``).

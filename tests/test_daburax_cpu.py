@@ -21,6 +21,11 @@ def test_frequencies():
     K.case_frequencies()
 
 
+def test_expert_block():
+    K.case_expert_block("cpu", F32)
+    K.case_expert_block("cpu", F32, W=32, ff=8, E=3, ident=0, top=1, cnt=1, keep=1, shared=0)
+
+
 def test_retention_scan_interleaved_pairs_whole_head():
     K.case_retention_scan("cpu", F32, H=2, D=8, Dv=12, dims=8, half=False, T=40)
 
@@ -30,7 +35,8 @@ def test_sink_needle(size):
     K.case_sink_needle("cpu", F32, size=size, n=120)
 
 
-@pytest.mark.parametrize("cfg", [C.config_a, C.config_b, C.config_c], ids=lambda f: f.__name__)
+@pytest.mark.parametrize("cfg", [C.config_a, C.config_b, C.config_c, C.config_d],
+                         ids=lambda f: f.__name__)
 def test_layers(cfg):
     K.case_layers("cpu", F32, cfg)
 
@@ -69,7 +75,7 @@ def test_every_tensor_has_a_place():
     by the checkpoint, and an unknown name is refused."""
     from enterprise_inference_amd.config import ModelConfig
     from enterprise_inference_amd.models import get_model_class
-    for cfg in (C.config_a(), C.config_b(), C.config_c()):
+    for cfg in (C.config_a(), C.config_b(), C.config_c(), C.config_d()):
         model = get_model_class("Daburax")(ModelConfig.from_hf_dict(cfg), dtype=F32)
         W = C.random_weights(cfg, 1)
         loaded = set(model.load_weights(W.items()))

@@ -80,6 +80,20 @@ def test_sink_needle(shape, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [
+    # W, ff, experts, identity, top, groups, keep, shared ff, tokens
+    (46, 20, 6, 2, 3, 4, 2, 12, 21),            # per-expert form
+    (128, 64, 6, 2, 2, 2, 1, 64, 40),           # grouped matrix-core form
+    (256, 256, 14, 2, 2, 4, 2, 256, 32),        # grouped weight-streaming form (decode-sized)
+    (256, 256, 3, 1, 2, 2, 1, 0, 700),          # many rows per expert
+    (512, 128, 8, 0, 2, 1, 1, 128, 9),
+], ids=lambda s: "-".join(map(str, s)))
+def test_expert_block(shape, dtype):
+    W, ff, E, ident, top, cnt, keep, shared, T = shape
+    K.case_expert_block("cuda", dtype, W, ff, E, ident, top, cnt, keep, shared, T)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("cfg", [C.config_a, C.config_b, C.config_c], ids=lambda f: f.__name__)
 def test_layers(cfg, dtype):
     K.case_layers("cuda", dtype, cfg)
@@ -95,6 +109,11 @@ def test_schedules(cfg, dtype):
 def test_schedules_pages_of_32(dtype):
     """Pages of 32 tokens: the bf16 run takes the matrix-core attention form end to end."""
     K.case_schedules("cuda", dtype, C.config_c, seed=3, block_size=32)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_schedules_odd_shared_row(dtype):
+    K.case_schedules("cuda", dtype, C.config_d, seed=5, block_size=32)
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
