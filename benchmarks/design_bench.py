@@ -153,18 +153,18 @@ def daburax_config(z: dict) -> dict:
            "router": {"experts": z["experts"] - 2, "identity": 2, "top": z["top"],
                       "groups": {"count": 4, "keep": 2}}}
     ret = {"type": "retention", "mlp": mlp,
-           "mixer": {"heads": H, "dim": D, "vdim": D, "rot": {"base": 1e6, "dims": D},
-                     "decay": [1.0 - 2.0 ** (-5 - 4 * i / H) for i in range(H)]}}
+           "mixer": {"heads": H, "dim": D, "vdim": D, "rot": {"base": 1e4, "dims": D},
+                     "decay": [1.0 - 2.0 ** (-4 - 6 * i / H) for i in range(H)]}}
     par = {"type": "parallel", "mlp": mlp,
            "mixer": {"left": {"heads": H, "kv_heads": max(1, H // 4), "dim": D, "vdim": D,
                               "scale": D ** -0.5,
-                              "rot": {"base": 5e4, "dims": D // 2, "scaling": {"factor": 2.0}}},
-                     "right": {"heads": H // 2, "dim": D, "vdim": D, "gate_cap": 12.0},
+                              "rot": {"base": 5e5, "dims": D // 2, "scaling": {"factor": 4.0}}},
+                     "right": {"heads": H // 2, "dim": D, "vdim": D, "gate_cap": 15.0},
                      "left_scale": 1.0, "right_scale": 1.0}}
     return {"architecture": "Daburax", "vocab": z["vocab"], "width": z["width"],
-            "norm": {"eps": 1e-5}, "residual_mult": 0.5, "streams": z["streams"],
+            "norm": {"eps": 1e-5}, "residual_mult": 0.7, "streams": z["streams"],
             "embedding": {"scale": z["width"] ** 0.5,
-                          "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+                          "bigram": {"buckets": 65521, "mul_prev": 1009, "mul_cur": 8191}},
             "layers": [ret, ret, par] * (z["layers"] // 3)}
 
 
@@ -637,10 +637,10 @@ def daburax_kernel_rates(a) -> int:
             cu = torch.arange(0, T + 1, per, dtype=torch.int32, device=dev)
             pos = (torch.arange(T, dtype=torch.int32, device=dev) % per) + (5 if per == 1 else 0)
             fused = (torch.randn(T, 4 * Hh * D + 2 * Hh, device=dev) * 0.3).to(bf)
-            inv, _ = rotary_frequencies(D, 1e6, None, dev)
+            inv, _ = rotary_frequencies(D, 1e4, None, dev)
             for mode in ("decay", "exp_gates"):
                 spec = LS.ScanSpec(Hh, D, D, mode,
-                                   decay=torch.full((Hh,), 0.97, device=dev), cap=12.0,
+                                   decay=torch.full((Hh,), 0.97, device=dev), cap=15.0,
                                    inv_freq=inv if mode == "decay" else None,
                                    rot_dims=D if mode == "decay" else 0, kscale=D ** -0.5,
                                    gate_act="silu" if mode == "decay" else "sigmoid", eps=1e-5)

@@ -81,7 +81,7 @@ def config_c():
     """Sizes in multiples of the matrix-core tiles, four streams, heads of 32 .. 64 with value
     sizes that differ from the key sizes, expert sizes that take the grouped expert kernels."""
     return {"architecture": "Daburax", "vocab": 160, "width": 128, "norm": {"eps": 1e-5},
-            "residual_mult": 0.5, "streams": 4,
+            "residual_mult": 0.6, "streams": 4,
             "embedding": {"scale": 4.0, "bigram": {"buckets": 101, "mul_prev": 13, "mul_cur": 29}},
             "layers": [moe(par(lh=4, lg=2, ld=32, lv=64, ldims=16, lbase=20000.0, factor=2.0,
                                lscale=0.15, rh=2, rd=64, rv=32, cap=10.0, ls=1.2, rs=0.9),
@@ -90,7 +90,7 @@ def config_c():
                                base=100000.0), experts=4, top=2, identity=0, count=2, keep=2,
                            ff=64, shared=128),
                        moe(par(lh=8, lg=1, ld=64, lv=16, ldims=64, factor=0, lscale=0.1, rh=4,
-                               rd=32, rv=32, cap=12.0, ls=0.7, rs=1.4), experts=0)]}
+                               rd=32, rv=32, cap=11.0, ls=0.7, rs=1.4), experts=0)]}
 
 
 def config_d():
