@@ -679,10 +679,13 @@ def daburax_kernel_rates(a) -> int:
     nb, nbd = T // bs, B * L // bs
     pos = torch.arange(T, dtype=torch.int32, device=dev)
     bt = torch.arange(nb, dtype=torch.int32, device=dev)[None]
+    # (the step's work list as the model runner builds it: latest query blocks first)
+    wl = A.build_prefill_work([T], WA.MFMA_QB)
     md = A.AttentionMetadata(
         num_decode=0, num_prefill_tokens=T, slot_mapping=pos, positions=pos,
         prefill_block_tables=bt, prefill_seq_lens=i32([T]), prefill_cu_q=i32([0, T]),
-        prefill_q_lens=[T])
+        prefill_q_lens=[T], prefill_work=i32(wl), prefill_n_work=len(wl) // 2,
+        prefill_qblock=WA.MFMA_QB)
     btd = torch.arange(nbd, dtype=torch.int32, device=dev).view(B, L // bs)
     posd = torch.full((B,), L - 1, dtype=torch.int32, device=dev)
     mdd = A.AttentionMetadata(num_decode=B, num_prefill_tokens=0, slot_mapping=posd,

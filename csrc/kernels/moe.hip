@@ -811,38 +811,50 @@ EIA_API int eia_moe_combine_postnorm(const void* h2, long ldh, const float* w, c
 // ---------------------------------------------------------------------------------------------
 // End of an expert block with identity experts and a gated always-on expert, one launch:
 //   out[t] = routed[t] + ident_w[t] * x[t] + sgate[t] * shared[t]
-// (ident_w, shared and sgate are nullable; sgate == nullptr with shared: weight 1).  fp32 sum,
-// stored in the activation type T.
+// (ident_w, shared and sgate are nullable; sgate == nullptr with shared: weight 1; the shared
+// rows are stored, or still the fp32 split-K partials spart [ssk, T, H] of their GEMM).  fp32
+// sum, stored in the activation type T.
 template <typename T>
 __global__ void __launch_bounds__(256)
 moe_finish_kernel(const T* __restrict__ routed, long ldr, const T* __restrict__ x, long ldx,
                   const float* __restrict__ ident_w, const T* __restrict__ shared, long lds_,
+                  const float* __restrict__ spart, int ssk, long spstride,
                   const float* __restrict__ sgate, T* __restrict__ out, long ldo, int H) {
   const long t = blockIdx.x;
   const float iw = ident_w ? ident_w[t] : 0.f;
-  const float sg = shared ? (sgate ? sgate[t] : 1.f) : 0.f;
+  const float sg = (shared || spart) ? (sgate ? sgate[t] : 1.f) : 0.f;
   for (int c = threadIdx.x; c < H; c += blockDim.x) {
     float v = ld_f32<T>(routed + t * ldr, c);
     if (ident_w) v += iw * ld_f32<T>(x + t * ldx, c);
-    if (shared) v += sg * ld_f32<T>(shared + t * lds_, c);
+    if (shared) {
+      v += sg * ld_f32<T>(shared + t * lds_, c);
+    } else if (spart) {
+      float sv = 0.f;
+      for (int z = 0; z < ssk; ++z) sv += spart[z * spstride + t * H + c];
+      v += sg * sv;
+    }
     st_f32<T>(out + t * ldo, c, v);
   }
 }
 
 EIA_API int eia_moe_finish(const void* routed, long ldr, const void* x, long ldx,
                            const float* ident_w, const void* shared, long lds_,
-                           const float* sgate, void* out, long ldo, int T, int H, int is_bf16,
-                           hipStream_t st) {
-  if (T < 0 || H < 1 || !routed || !out || (ident_w && !x)) return EIA_BAD_SHAPE;
+                           const float* spart, int ssk, const float* sgate, void* out, long ldo,
+                           int T, int H, int is_bf16, hipStream_t st) {
+  if (T < 0 || H < 1 || !routed || !out || (ident_w && !x) || (shared && spart) ||
+      (spart && ssk < 1))
+    return EIA_BAD_SHAPE;
   if (T == 0) return EIA_OK;
   const int threads = H >= 1024 ? 256 : (H >= 512 ? 128 : 64);
   if (is_bf16)
     hipLaunchKernelGGL((moe_finish_kernel<bf16_t>), dim3(T), dim3(threads), 0, st,
                        (const bf16_t*)routed, ldr, (const bf16_t*)x, ldx, ident_w,
-                       (const bf16_t*)shared, lds_, sgate, (bf16_t*)out, ldo, H);
+                       (const bf16_t*)shared, lds_, spart, ssk, (long)T * H, sgate, (bf16_t*)out,
+                       ldo, H);
   else
     hipLaunchKernelGGL((moe_finish_kernel<float>), dim3(T), dim3(threads), 0, st,
                        (const float*)routed, ldr, (const float*)x, ldx, ident_w,
-                       (const float*)shared, lds_, sgate, (float*)out, ldo, H);
+                       (const float*)shared, lds_, spart, ssk, (long)T * H, sgate, (float*)out,
+                       ldo, H);
   EIA_LAUNCH_CHECK();
 }

@@ -77,7 +77,7 @@ _SIGNATURES = {
     "eia_moe_route_grouped": [P, L, P, I, I, I, I, I, I, F, P, P, IP, I, I, I, I, P, I, P, P, P, S],
     "eia_linear_scan": [P, L, I, I, I, I, I, I, P, P, I, I, F, F, F, F, P, P, P, P, IP, IP, IP, IP,
                         P, L, F, I, I, I, I, I, I, I, S],
-    "eia_moe_finish": [P, L, P, L, P, P, L, P, P, L, I, I, I, S],
+    "eia_moe_finish": [P, L, P, L, P, P, L, P, I, P, P, L, I, I, I, S],
     "eia_linear_scan_chunked": [P, L, I, I, I, I, I, I, P, P, I, I, F, F, F, F, P, P, P, P, IP, IP,
                                 IP, P, L, F, I, I, I, I, I, I, I, IP, IP, I, P, P, P, P, P, P, S],
     "eia_hyper_step": [P, I, I, P, L, P, I, P, P, P, F, P, P, F, P, L, F, I, I, S],

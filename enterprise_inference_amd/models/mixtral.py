@@ -359,10 +359,9 @@ class GroupLimitedMoE(nn.Module):
         tw, ids = r[0], r[1]
         ident_w, sgate = (r[2], r[3]) if len(r) == 4 else (None, None)
         routed = moe_ops.fused_moe(x, self.w13, self.w2, tw, ids, (0, self.E), act=self.act)
-        shared = None
-        if self.shared is not None:
-            shared = self.shared(x)
-            shared = shared.materialize() if hasattr(shared, "materialize") else shared
+        # (the shared expert's down projection may hand on split-K partials: summed in the
+        # block's final launch)
+        shared = self.shared(x) if self.shared is not None else None
         return moe_ops.finish_gated(routed, x, ident_w, shared, sgate)
 
 

@@ -542,7 +542,17 @@ def finish_gated(routed: torch.Tensor, x: torch.Tensor, ident_w: Optional[torch.
                  shared: Optional[torch.Tensor], sgate: Optional[torch.Tensor]) -> torch.Tensor:
     """End of an expert block with identity experts and a gated shared expert, summed in fp32
     (moe.hip moe_finish_kernel, one launch):
-    routed + ident_w[:, None] * x + sgate[:, None] * shared  -> [T, H] in x's dtype."""
+    routed + ident_w[:, None] * x + sgate[:, None] * shared  -> [T, H] in x's dtype.
+    ``shared`` may be a ``gemm.SplitK`` without bias (fp32 partial sums of the shared expert's
+    down projection), summed here."""
+    from .gemm import SplitK
+    spart = None
+    if isinstance(shared, SplitK):
+        if (use_hip(x) and shared.bias is None and shared.part.is_contiguous()
+                and shared.M == x.shape[0] and shared.N == x.shape[1]):
+            spart, shared = shared, None
+        else:
+            shared = shared.materialize().to(x.dtype)
     if not use_hip(x):
         y = routed.float()
         if ident_w is not None:
@@ -562,6 +572,8 @@ def finish_gated(routed: torch.Tensor, x: torch.Tensor, ident_w: Optional[torch.
     out = torch.empty(T, H, dtype=dt, device=x.device)
     check(lib().eia_moe_finish(ptr(routed), routed.stride(0), ptr(x), x.stride(0), ptr(ident_w),
                                ptr(shared), shared.stride(0) if shared is not None else 0,
+                               ptr(spart.part) if spart is not None else None,
+                               spart.sk if spart is not None else 0,
                                ptr(sgate), ptr(out), out.stride(0), T, H,
                                1 if dt == torch.bfloat16 else 0, stream(x)), "moe_finish")
     return out
