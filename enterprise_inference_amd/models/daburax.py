@@ -310,10 +310,10 @@ class DaburaxForCausalLM(nn.Module):
         around zero, matrices N(0, 1/fan_in), stream constants near the plain residual sum,
         small sinks and gate biases."""
         import zlib
-        for mod in self.modules():
+        for mname, mod in self.named_modules():
             if isinstance(mod, FusedProjection):
                 g = torch.Generator(device=mod.weight.device)
-                g.manual_seed(seed * 1000003 + zlib.crc32(repr(sorted(mod.offsets)).encode()))
+                g.manual_seed(seed * 1000003 + zlib.crc32(mname.encode()))
                 mod.init_random(g)
         for name, p in self.named_parameters():
             if name.endswith(("proj.weight", "proj.bias")) and ".mix." in name:
